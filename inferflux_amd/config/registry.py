@@ -2,8 +2,8 @@
 
 An architecture is registered as (config class, plan builder): the config class parses
 config.json, the plan builder turns the typed config into a ``ModelPlan`` (a list of
-layers made of parts, and the order they run in).  Lookup goes by ``model_type`` and then
-by ``architectures[0]``, the order the reference uses
+layers made of parts, and the order they run in).  Lookup goes by ``model_type``, then by
+``architectures[0]`` (and last by a single ``architecture`` string), the order the reference uses
 (runtime/backends/cuda/inferflux_cuda_executor.cpp:576-583); an unknown name is an error
 that lists what is registered (the reference returns nullptr and logs "Unsupported
 model_type", runtime/backends/cuda/native/model_forward_factory.cpp:46-60).
@@ -50,6 +50,9 @@ def resolve_architecture(d: Mapping[str, Any]) -> Tuple[Type[ModelConfig], Calla
     archs = d.get("architectures")
     if isinstance(archs, list) and archs and isinstance(archs[0], str):
         candidates.append(archs[0])
+    one = d.get("architecture")          # files that name their design in one string
+    if isinstance(one, str) and one:
+        candidates.append(one)
     if not candidates:
         raise ConfigError("config.json names neither 'model_type' nor 'architectures'")
     for c in candidates:

@@ -1,4 +1,4 @@
-// Plain attention over the paged cache: any head size up to 256, float or bf16 storage, float
+// Plain attention over the paged cache: any head size up to 640, float or bf16 storage, float
 // math.  One wave per (query row, query head): each lane scores one key of a 64-key tile, the
 // wave takes the tile's maximum and sum, then every lane accumulates its output elements over
 // the tile's keys in ascending order.  Tiles are aligned to absolute key positions (multiples of
@@ -17,7 +17,7 @@
 
 IFX_DEFINE_LAST_ERROR()
 
-#define MAX_D 256
+#define MAX_D 640
 #define DC (MAX_D / WAVE)
 #define WAVES_PER_BLOCK 4
 

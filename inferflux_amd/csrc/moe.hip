@@ -1,0 +1,196 @@
+// Mixture of experts: the router and the experts' products for rows that each choose their own experts.
+//
+//   ifx_moe_route     z = W_r h in float, score s = sigmoid(z) (or softmax over the experts), choice of `top` experts
+//                     among those of the best `keep` of `groups` equal groups of neighbouring experts (a group's
+//                     score: the sum of its `group_top` largest scores); the weights are the chosen scores as they
+//                     are or divided by their sum.  Writes ids [T][top] (int32) and weights [T][top] (float), in
+//                     descending order of score, the lower index first among equals.
+//   ifx_moe_gate_up   a[t][j][:] = silu(Wg[e] h_t) * (Wu[e] h_t) for e = ids[t][j]       (Wg, Wu [E][ff][K])
+//   ifx_moe_down      out[t][:] = sum_j weights[t][j] * Wd[e_j] a[t][j][:]              (Wd [E][N][ff])
+//
+// The two product kernels read the expert of every (row, choice) from device memory, so their grid depends on the
+// step's layout alone.  One wave forms one output element at a time (lanes across k, the fixed-order sum of
+// common.h), so a row's result does not depend on what shares its batch.  They are the path of the 32-bit mode and of
+// steps of few rows; bfloat16 steps of many rows take the grouped matrix-core product (moe_grouped.hip).
+#include "common.h"
+
+IFX_DEFINE_LAST_ERROR()
+
+#define MAX_EXPERTS 1024
+#define MAX_TOP 32
+
+struct RouteArgs {
+  const void* h; const void* w; int* ids; float* weights;
+  int T, K, E, top, groups, keep, group_top, softmax, renorm;
+  float scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(RouteArgs a) {
+  __shared__ float s[MAX_EXPERTS];       // scores
+  __shared__ float gs[MAX_EXPERTS];      // group scores (-1: a group that is shut out)
+  __shared__ float red[16];
+  const size_t t = blockIdx.x;
+  const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
+  const T* h = (const T*)a.h + t * a.K;
+  const T* w = (const T*)a.w;
+  for (int e = wid; e < a.E; e += nw) {
+    float z = 0.f;
+    for (int k = lane; k < a.K; k += WAVE) z = fmaf(to_f(h[k]), to_f(w[(size_t)e * a.K + k]), z);
+    z = wave_sum(z);
+    if (lane == 0) s[e] = z;
+  }
+  __syncthreads();
+  if (a.softmax) {
+    float m = -INFINITY;
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) m = fmaxf(m, s[e]);
+    m = block_max(m, red);
+    float l = 0.f;
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) l += expf(s[e] - m);
+    l = block_sum(l, red);
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] = expf(s[e] - m) / l;
+  } else {
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] = 1.0f / (1.0f + expf(-s[e]));
+  }
+  __syncthreads();
+  // The choice is a few hundred comparisons: one thread makes it.
+  if (threadIdx.x != 0) return;
+  const int per = a.E / a.groups;
+  if (a.keep < a.groups) {
+    for (int g = 0; g < a.groups; ++g) {
+      // sum of the group's group_top largest scores (scores lie in (0, 1): -1 marks one taken)
+      float sum = 0.f;
+      int taken[8];
+      for (int r = 0; r < a.group_top && r < per; ++r) {
+        int best = -1;
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          bool used = false;
+          for (int q = 0; q < r; ++q) used |= taken[q] == e;
+          if (!used && (best < 0 || s[e] > s[best])) best = e;
+        }
+        taken[r] = best;
+        sum += s[best];
+      }
+      gs[g] = sum;
+    }
+    // all but the best `keep` groups are shut out
+    for (int r = 0; r < a.groups - a.keep; ++r) {
+      int worst = -1;
+      for (int g = a.groups - 1; g >= 0; --g)          // among equals the higher index goes first
+        if (gs[g] >= 0.f && (worst < 0 || gs[g] < gs[worst])) worst = g;
+      gs[worst] = -1.f;
+    }
+  } else {
+    for (int g = 0; g < a.groups; ++g) gs[g] = 0.f;
+  }
+  int chosen[MAX_TOP];
+  float total = 0.f;
+  for (int r = 0; r < a.top; ++r) {
+    int best = -1;
+    for (int e = 0; e < a.E; ++e) {
+      if (gs[e / per] < 0.f) continue;
+      bool used = false;
+      for (int q = 0; q < r; ++q) used |= chosen[q] == e;
+      if (!used && (best < 0 || s[e] > s[best])) best = e;
+    }
+    chosen[r] = best;
+    total += s[best];
+  }
+  for (int r = 0; r < a.top; ++r) {
+    a.ids[t * a.top + r] = chosen[r];
+    a.weights[t * a.top + r] = (a.renorm ? s[chosen[r]] / total : s[chosen[r]]) * a.scale;
+  }
+}
+
+extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, int* ids, float* weights, int T, int K, int E, int top,
+                             int groups, int keep, int group_top, int softmax, int renorm, float scale, void* stream) {
+  IFX_REQUIRE(T >= 0 && K > 0 && E > 0 && E <= MAX_EXPERTS, "moe_route: %d experts (at most %d), K=%d", E, MAX_EXPERTS, K);
+  IFX_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups, "moe_route: %d experts in %d groups of which %d are kept", E, groups, keep);
+  IFX_REQUIRE(group_top > 0 && group_top <= 8, "moe_route: a group's score sums its %d largest (1-8)", group_top);
+  IFX_REQUIRE(top > 0 && top <= MAX_TOP && top <= keep * (E / groups), "moe_route: top %d of %d x %d experts", top, keep, E / groups);
+  if (T == 0) return 0;
+  RouteArgs a{h, w, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale};
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(256), 0, s, a);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(256), 0, s, a);
+  else IFX_FAIL("moe_route: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+#define ROWS_PER_WAVE 4
+#define WAVES 4
+
+template <typename T>
+__global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ wg,
+                                                                   const T* __restrict__ wu, const int* __restrict__ ids,
+                                                                   T* __restrict__ act, int K, int ff, int top) {
+  const size_t item = blockIdx.x;                 // (row, choice)
+  const size_t t = item / top;
+  const int e = ids[item];
+  const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const T* x = h + t * K;
+  const int i0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
+  for (int i = i0; i < i0 + ROWS_PER_WAVE && i < ff; ++i) {
+    const T* g = wg + ((size_t)e * ff + i) * K;
+    const T* u = wu + ((size_t)e * ff + i) * K;
+    float sg = 0.f, su = 0.f;
+    for (int k = lane; k < K; k += WAVE) {
+      const float xv = to_f(x[k]);
+      sg = fmaf(xv, to_f(g[k]), sg);
+      su = fmaf(xv, to_f(u[k]), su);
+    }
+    sg = wave_sum(sg);
+    su = wave_sum(su);
+    if (lane == 0) act[item * ff + i] = from_f<T>(sg / (1.0f + expf(-sg)) * su);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restrict__ act, const T* __restrict__ wd,
+                                                                const int* __restrict__ ids, const float* __restrict__ weights,
+                                                                T* __restrict__ out, int N, int ff, int top) {
+  const size_t t = blockIdx.x;
+  const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int n0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
+  for (int n = n0; n < n0 + ROWS_PER_WAVE && n < N; ++n) {
+    float y = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const int e = ids[t * top + j];
+      const T* w = wd + ((size_t)e * N + n) * ff;
+      const T* a = act + (t * top + j) * ff;
+      float s = 0.f;
+      for (int k = lane; k < ff; k += WAVE) s = fmaf(to_f(a[k]), to_f(w[k]), s);
+      y = fmaf(weights[t * top + j], wave_sum(s), y);
+    }
+    if (lane == 0) out[t * N + n] = from_f<T>(y);
+  }
+}
+
+extern "C" int ifx_moe_gate_up(const void* h, const void* wg, const void* wu, const int* ids, void* act, int dtype, int T, int K,
+                               int ff, int top, void* stream) {
+  IFX_REQUIRE(T >= 0 && K > 0 && ff > 0 && top > 0, "moe_gate_up: bad sizes T=%d K=%d ff=%d top=%d", T, K, ff, top);
+  if (T == 0) return 0;
+  const dim3 grid((unsigned)T * top, (ff + WAVES * ROWS_PER_WAVE - 1) / (WAVES * ROWS_PER_WAVE));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)h, (const float*)wg, (const float*)wu, ids, (float*)act, K, ff, top);
+  else if (dtype == DT_BF16)
+    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)h, (const bf16_t*)wg, (const bf16_t*)wu, ids, (bf16_t*)act, K, ff, top);
+  else IFX_FAIL("moe_gate_up: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+extern "C" int ifx_moe_down(const void* act, const void* wd, const int* ids, const float* weights, void* out, int dtype, int T,
+                            int N, int ff, int top, void* stream) {
+  IFX_REQUIRE(T >= 0 && N > 0 && ff > 0 && top > 0, "moe_down: bad sizes T=%d N=%d ff=%d top=%d", T, N, ff, top);
+  if (T == 0) return 0;
+  const dim3 grid(T, (N + WAVES * ROWS_PER_WAVE - 1) / (WAVES * ROWS_PER_WAVE));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)act, (const float*)wd, ids, weights, (float*)out, N, ff, top);
+  else if (dtype == DT_BF16)
+    hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)act, (const bf16_t*)wd, ids, weights, (bf16_t*)out, N, ff, top);
+  else IFX_FAIL("moe_down: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}

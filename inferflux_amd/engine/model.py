@@ -123,6 +123,8 @@ class Model:
                 residual, pending = block.forward(residual, pending, ctx, storage.binding(i), following=following)
             else:
                 residual, pending = block.forward(residual, pending, ctx, storage.binding(i))
+        if getattr(pending, "in_stream", False):     # (a block's hand-over to its like; the stream holds everything)
+            pending = None
         if ctx.n_logit_rows == 0:
             logits = torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=residual.device)
         else:

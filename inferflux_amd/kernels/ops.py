@@ -52,6 +52,9 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("sampling", ())
     yield ("gemm_bf16", ())
     yield ("gemm_wide", ())
+    yield ("layernorm", ())
+    yield ("latent", ())
+    yield ("moe", ())
     yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
@@ -236,6 +239,155 @@ def swiglu(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
     _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, P),
           gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, _stream())
+    return out
+
+
+def _delta_args(delta, shape, name):
+    """(pointer, dtype code, slices, elements between slices) of a tensor or of a product left as ``SliceSums``."""
+    if isinstance(delta, SliceSums):
+        _check(delta.parts, name, (None, *shape), torch.float32)
+        return delta.parts.data_ptr(), DT_F32, delta.parts.shape[0], delta.parts[0].numel()
+    _check(delta, name, shape)
+    return delta.data_ptr(), _dt(delta), 1, 0
+
+
+def layernorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+              rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Layer norm with a weight and no bias of the rows of ``x`` [T, H] (float32 or bfloat16), in float:
+    (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight.  A ``delta`` (a tensor or ``SliceSums``) is added first,
+    and written back into ``x`` unless ``rows`` (int32 [R]) picks the rows to normalise."""
+    _check(x, "x", (None, None))
+    T, H = x.shape
+    _check(weight, "weight", (H,))
+    dp, dd, n_slices, stride = (0, 0, 1, 0) if delta is None else _delta_args(delta, (T, H), "delta")
+    n = T
+    if rows is not None:
+        _check(rows, "rows", (None,), torch.int32)
+        n = rows.shape[0]
+    out = torch.empty((n, H), dtype=out_dtype, device=x.device)
+    _call(load_module("layernorm"), "ifx_layernorm", (P, I, P, I, I, LL, P, I, P, I, P, I, I, F, P),
+          x.data_ptr(), _dt(x), dp, dd, n_slices, stride, weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype],
+          _ptr(rows), n, H, float(eps), _stream())
+    return out
+
+
+def add_layernorm(stream: torch.Tensor, delta, weight: torch.Tensor, eps: float,
+                  cast_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """``stream`` [T, H] (float32) += layer norm (weight, no bias) of ``delta`` [T, H] (a tensor or ``SliceSums``), in
+    place.  With ``cast_dtype`` the new stream rounded to that type is returned as well (what a sub-block that reads
+    the stream itself takes as its input); with float32 that is the stream."""
+    _check(stream, "stream", (None, None), torch.float32)
+    T, H = stream.shape
+    _check(weight, "weight", (H,))
+    dp, dd, n_slices, stride = _delta_args(delta, (T, H), "delta")
+    cast = torch.empty((T, H), dtype=cast_dtype, device=stream.device) if cast_dtype not in (None, torch.float32) else None
+    _call(load_module("layernorm"), "ifx_add_layernorm", (P, P, I, I, LL, P, I, P, I, I, I, F, P),
+          stream.data_ptr(), dp, dd, n_slices, stride, weight.data_ptr(), _dt(weight), _ptr(cast),
+          _DT[cast_dtype] if cast is not None else 0, T, H, float(eps), _stream())
+    return stream if cast_dtype == torch.float32 else cast
+
+
+def cast_rows(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 rows ``x`` rounded to ``dtype`` (bfloat16)."""
+    _check(x, "x", None, torch.float32)
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _call(load_module("layernorm"), "ifx_cast_rows", (P, P, I, LL, P), x.data_ptr(), out.data_ptr(), _DT[dtype], x.numel(), _stream())
+    return out
+
+
+def latent_finish(y, q_norm: Optional[torch.Tensor], kv_norm: torch.Tensor, eps: float, cos: Optional[torch.Tensor],
+                  sin: Optional[torch.Tensor], rot_dims: int, slots: Optional[torch.Tensor], q_rank: int, kv_rank: int,
+                  rot_dim: int, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int,
+                  dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """What follows the down projections of attention through a latent.  ``y`` [T, q_rank + kv_rank + rot_dim] (a
+    tensor or ``SliceSums``) holds per row the query latent, the key/value latent and the shared rotated key part.
+    Returns the query latent under its RMS norm (weight ``q_norm``) [T, q_rank] (None when ``q_rank`` is 0); with
+    ``slots`` (int32 [T] = page * page_size + offset) the key/value latent under its RMS norm (``kv_norm``) and the
+    key part, its first ``rot_dims`` elements turned by the table ``cos`` / ``sin`` [T, rot_dims / 2], go into the
+    cache: K rows [latent | key part] (``k_cache`` [pages, 1, page_size, kv_rank + rot_dim]) and V columns
+    (``v_cache`` [pages, 1, kv_rank, page_size])."""
+    width = q_rank + kv_rank + rot_dim
+    T = y.shape[0]
+    yp, yd, n_slices, stride = _delta_args(y, (T, width), "y")
+    if q_rank:
+        _check(q_norm, "q_norm", (q_rank,), kv_norm.dtype)
+    _check(kv_norm, "kv_norm", (kv_rank,))
+    if rot_dims:
+        _check(cos, "cos", (T, rot_dims // 2), torch.float32)
+        _check(sin, "sin", (T, rot_dims // 2), torch.float32)
+    if slots is not None:
+        _check(slots, "slots", (T,), torch.int32)
+        _check(k_cache, "k_cache", (None, 1, page_size, kv_rank + rot_dim), dtype)
+        _check(v_cache, "v_cache", (k_cache.shape[0], 1, kv_rank, page_size), dtype)
+    cq = torch.empty((T, q_rank), dtype=dtype, device=kv_norm.device) if q_rank else None
+    _call(load_module("latent"), "ifx_latent_finish", (P, I, I, LL, P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P),
+          yp, yd, n_slices, stride, _ptr(q_norm), kv_norm.data_ptr(), _dt(kv_norm), _ptr(cos) if rot_dims else 0,
+          _ptr(sin) if rot_dims else 0, rot_dims, _ptr(slots), _ptr(cq), _ptr(k_cache) if slots is not None else 0,
+          _ptr(v_cache) if slots is not None else 0, _DT[dtype], T, q_rank, kv_rank, rot_dim, page_size, float(eps), _stream())
+    return cq
+
+
+def headwise(x: torch.Tensor, weight: torch.Tensor, n_heads: int, x_head: int, tail: int = 0,
+             cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dims: int = 0) -> torch.Tensor:
+    """A product per head: out[t, h, :N] = ``weight``[h] x[t, h] with ``weight`` [H, N, K] and head h's input the K
+    elements of row t of ``x`` [T, >= H * x_head] from h * x_head on.  The ``tail`` elements that follow a head's K
+    inputs are appended to its output, the first ``rot_dims`` of them turned by the table ``cos`` / ``sin``
+    [T, rot_dims / 2] in split-half pairs.  Returns [T, H, N + tail] in x's type; sums in float."""
+    _check(x, "x", (None, None))
+    T = x.shape[0]
+    _check(weight, "weight", (n_heads, None, None), x.dtype)
+    _, N, K = weight.shape
+    if x_head < K + tail or x.shape[1] < (n_heads - 1) * x_head + K + tail:
+        raise KernelError(f"headwise: {n_heads} heads of {K} + {tail} inputs, {x_head} apart, do not fit rows of {x.shape[1]}")
+    if rot_dims:
+        _check(cos, "cos", (T, rot_dims // 2), torch.float32)
+        _check(sin, "sin", (T, rot_dims // 2), torch.float32)
+    out = torch.empty((T, n_heads, N + tail), dtype=x.dtype, device=x.device)
+    _call(load_module("latent"), "ifx_headwise", (P, P, P, I, I, I, I, I, I, I, I, P, P, I, P),
+          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _dt(x), T, n_heads, K, N, x.shape[1], x_head, tail,
+          _ptr(cos) if rot_dims else 0, _ptr(sin) if rot_dims else 0, rot_dims, _stream())
+    return out
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, groups: int = 1, keep_groups: int = 1, group_top: int = 2,
+              softmax: bool = False, renormalize: bool = False, scale: float = 1.0):
+    """The router of a mixture of experts, in float: scores of ``router`` [E, K] times the rows of ``h`` [T, K] through a
+    sigmoid (or a softmax over the experts), the ``top`` highest among the experts of the best ``keep_groups`` of
+    ``groups`` equal groups of neighbours (a group scores the sum of its ``group_top`` highest).  Returns (ids int32
+    [T, top], weights float32 [T, top]): the chosen scores, divided by their sum with ``renormalize``, times ``scale``."""
+    _check(h, "h", (None, None))
+    T, K = h.shape
+    _check(router, "router", (None, K), h.dtype)
+    E = router.shape[0]
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, I, I, I, I, I, I, I, I, I, F, P),
+          h.data_ptr(), router.data_ptr(), _dt(h), ids.data_ptr(), weights.data_ptr(), T, K, E, top, groups, keep_groups,
+          group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _stream())
+    return ids, weights
+
+
+def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
+                     weights: torch.Tensor) -> torch.Tensor:
+    """sum_j weights[t, j] * down[e] (silu(gate[e] h_t) * (up[e] h_t)), e = ids[t, j], row by row: every (row, choice)
+    streams its expert's weights (``gate`` / ``up`` [E, ff, K], ``down`` [E, N, ff], in h's type).  Returns [T, N]."""
+    _check(h, "h", (None, None))
+    T, K = h.shape
+    _check(gate, "gate", (None, None, K), h.dtype)
+    E, ff, _ = gate.shape
+    _check(up, "up", (E, ff, K), h.dtype)
+    _check(down, "down", (E, None, ff), h.dtype)
+    N = down.shape[1]
+    top = ids.shape[1]
+    _check(ids, "ids", (T, top), torch.int32)
+    _check(weights, "weights", (T, top), torch.float32)
+    mod = load_module("moe")
+    act = torch.empty((T, top, ff), dtype=h.dtype, device=h.device)
+    _call(mod, "ifx_moe_gate_up", (P, P, P, P, P, I, I, I, I, I, P),
+          h.data_ptr(), gate.data_ptr(), up.data_ptr(), ids.data_ptr(), act.data_ptr(), _dt(h), T, K, ff, top, _stream())
+    out = torch.empty((T, N), dtype=h.dtype, device=h.device)
+    _call(mod, "ifx_moe_down", (P, P, P, P, P, I, I, I, I, I, P),
+          act.data_ptr(), down.data_ptr(), ids.data_ptr(), weights.data_ptr(), out.data_ptr(), _dt(h), T, N, ff, top, _stream())
     return out
 
 

@@ -6,6 +6,11 @@
 delta, and the norm that follows adds it to the float32 stream in the same kernel that
 normalises (the reference's ResidualAddRmsNorm, cuda_kernels.cu:617-671).
 
+"outnorm" puts the norms on the sub-blocks' outputs instead: x <- x + norm1(mixer(x)), then
+x <- x + norm2(ffn(x)); the sub-blocks read the stream itself (rounded to the activation type), and a layer may
+have no feed-forward.  Its norms are parts with ``add_to(stream, delta, cast_dtype)``, which adds the normed delta
+into the stream and returns the rounding that the next sub-block reads, all in one kernel.
+
 For steps of few rows a sub-block that can do so adds its output to the stream in its last product's
 epilogue and hands on the next norm's rows up to a factor per row (``ScaledRows``), which the sub-block
 after it applies to its first product's sums: the norm between them then needs no kernel.  Parts that
@@ -13,6 +18,9 @@ do not declare this are given plain tensors, and a plain delta is taken from the
 """
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from ..kernels.ops import ScaledRows
 from .base import Block, MixerBinding, StreamSink, build_part, register_part
 from .plan import LayerSpec
@@ -20,6 +28,8 @@ from .plan import LayerSpec
 
 def normed_for(norm, reader, residual, pending, ctx):
     """What ``reader`` is given: the norm of the stream plus ``pending``."""
+    if getattr(pending, "in_stream", False):     # rows some other arrangement prepared for its like: the stream holds everything
+        pending = None
     if isinstance(pending, ScaledRows):          # the delta is in the stream already
         accepts = getattr(reader, "accepts_scaled_rows", None)
         params = norm.rms_params()
@@ -76,3 +86,63 @@ class PreNormBlock(Block):
         t.enter("norm"); h = normed_for(self.norm_post, self.ffn, residual, delta, ctx); t.mark("norm")
         t.enter("ffn"); out = self._ffn(h, ctx, residual, following); t.mark("ffn")
         return residual, out
+
+
+@register_part("block", "outnorm")
+class OutputNormBlock(Block):
+    """x <- x + norm_in(mixer(x)); x <- x + norm_post(ffn(x)) (the second only if the layer has a feed-forward).  What
+    a sub-block reads, the stream in the activation type, is handed from block to block as ``pending`` wrapped in
+    ``StreamRows``, so that the kernel which adds a normed delta also writes the next reader's input."""
+    graph_safe = True
+
+    def __init__(self, layer: LayerSpec, hidden_size: int):
+        if layer.norm_in is None or layer.extra or (layer.ffn is None) != (layer.norm_post is None):
+            raise ValueError(f"layer {layer.prefix}: the outnorm block is a mixer with its norm and optionally a feed-forward with its norm")
+        self.prefix = layer.prefix
+        self.mixer = build_part("mixer", layer.mixer, hidden_size=hidden_size)
+        self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)
+        self.ffn = build_part("ffn", layer.ffn, hidden_size=hidden_size) if layer.ffn is not None else None
+        self.norm_post = build_part("norm", layer.norm_post, hidden_size=hidden_size) if layer.norm_post is not None else None
+        for n in (self.norm_in, self.norm_post):
+            if n is not None and not hasattr(n, "add_to"):
+                raise ValueError(f"layer {layer.prefix}: the outnorm block needs norms that can add to the stream (add_to)")
+
+    def children(self):
+        return tuple(p for p in (self.mixer, self.norm_in, self.ffn, self.norm_post) if p is not None)
+
+    def forward(self, residual, pending, ctx, binding: MixerBinding, following=None):
+        t = ctx.timer
+        if isinstance(pending, StreamRows) and pending.stream is residual:
+            h = pending.rows
+        else:
+            if pending is not None:                       # a delta some other arrangement left: it belongs to the stream
+                residual += pending.sum(torch.float32) if hasattr(pending, "parts") else pending.float()
+            h = residual if ctx.act_dtype == torch.float32 else ops.cast_rows(residual, ctx.act_dtype)
+        if t is not None:
+            t.enter("mixer")
+        delta = self.mixer.forward(h, ctx, binding)
+        if t is not None:
+            t.mark("mixer"); t.enter("norm")
+        h = self.norm_in.add_to(residual, delta, ctx.act_dtype)
+        if t is not None:
+            t.mark("norm")
+        if self.ffn is not None:
+            if t is not None:
+                t.enter("ffn")
+            delta = self.ffn.forward(h, ctx)
+            if t is not None:
+                t.mark("ffn"); t.enter("norm")
+            h = self.norm_post.add_to(residual, delta, ctx.act_dtype)
+            if t is not None:
+                t.mark("norm")
+        return residual, StreamRows(residual, h)
+
+
+class StreamRows:
+    """The stream rounded to the activation type (``rows``), valid for ``stream`` as it stands: what the next block
+    that reads the stream itself takes as its input.  Anyone else ignores it (the stream already holds everything)."""
+    __slots__ = ("stream", "rows")
+    in_stream = True          # nothing is left to add: a reader that has no use for the rows drops them
+
+    def __init__(self, stream, rows):
+        self.stream, self.rows = stream, rows

@@ -22,15 +22,17 @@ from .plan import ParamSpec
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02, tensor: Optional[str] = None):
+        """``tensor``: the table's full name in the model file where that is not ``<name>.weight``."""
         self.name, self.vocab_size, self.hidden_size, self.init_std = name, int(vocab_size), int(hidden_size), init_std
+        self.tensor = tensor or f"{name}.weight"
         self.table: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {f"{self.name}.weight": ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+        return {self.tensor: ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.table = tensors[f"{self.name}.weight"]
+        self.table = tensors[self.tensor]
 
     prepares_norm_rows = True
 
@@ -51,17 +53,20 @@ class LinearHead(Part):
 
     """``tied_to`` names the tensor (the embedding table) a tied head shares; None for its own."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02,
+                 tensor: Optional[str] = None):
+        """``tensor``: the weight's full name in the model file where that is not ``<name>.weight``."""
         self.name, self.vocab_size, self.hidden_size, self.tied_to, self.init_std = name, int(vocab_size), int(hidden_size), tied_to, init_std
+        self.tensor = tensor or f"{name}.weight"
         self.weight: Optional[ops.LinearWeight] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if self.tied_to:
             return {}
-        return {f"{self.name}.weight": ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+        return {self.tensor: ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = ops.prepare_linear(tensors[self.tied_to or f"{self.name}.weight"])
+        self.weight = ops.prepare_linear(tensors[self.tied_to or self.tensor])
 
     def accepts_scaled_rows(self, n_rows: int) -> bool:
         return ops.takes_scaled_rows(n_rows, self.weight)

@@ -1,0 +1,103 @@
+"""Attention through a latent: queries, keys and values are projected down to narrow latents first, and only the
+key/value latent and one shared rotated key part are cached.
+
+With H heads of ``dim`` unrotated and ``rot_dim`` rotated query/key dimensions, values of ``vdim``, a query latent of
+``q_rank`` and a key/value latent of ``kv_rank``:
+
+    c_q = rmsnorm(W_dq h) * g_q              q   = W_uq c_q, per head [q_n (dim) | q_r (rot_dim)]
+    c   = rmsnorm((W_dkv h)[:kv_rank]) * g_kv      k_r = (W_dkv h)[kv_rank:], one for all heads
+    per head: k_n = W_uk c, v = W_uv c
+    score(i, j) = (q_n(i) . k_n(j) + rot(q_r(i), i) . rot(k_r(j), j)) * scale,  j <= i (and within the window)
+    out = W_o [softmax-weighted sums of v, head by head]
+
+Neither k_n nor v is ever formed.  Since q_n . (W_uk c) = (W_uk^T q_n) . c, a head's query becomes
+[W_uk^T q_n | rot(q_r)] (kv_rank + rot_dim wide) and scores against the cached row [c | rot(k_r)], which all heads
+share; the weighted sum is taken over c itself and W_uv is applied to it afterwards.  To the paged attention kernels
+this is attention with one kv head whose keys are kv_rank + rot_dim and whose values kv_rank wide, so the cache, its
+pages, windows and block tables are those of every other attention layer (``CacheSpec`` with ``v_head_dim``), and a
+step's rows may be prompt portions and decoded tokens alike.
+
+Tensors (``<name>.``): dq [q_rank, H], dq.norm [q_rank], uq [heads (dim + rot_dim), q_rank], dkv [kv_rank + rot_dim, H],
+dkv.norm [kv_rank], uk [heads dim, kv_rank], uv [heads vdim, kv_rank], o [H, heads vdim].  The two down projections
+are one product (their weights are stacked at load), and W_uk is kept transposed per head.
+
+Norms, rotation angles, scores and softmax are computed in float whatever the activation type.
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from ..kernels.attention import paged_attention
+from .base import Mixer, MixerBinding, build_part, register_part
+from .ffn import concat_weights
+from .plan import CacheSpec, ParamSpec, PartSpec
+
+
+@register_part("mixer", "latent_attention")
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, name: str, hidden_size: int, n_heads: int, dim: int, rot_dim: int, v_dim: int, q_rank: int,
+                 kv_rank: int, scale: float, eps: float, position: PartSpec, window: Optional[int] = None,
+                 init_std: float = 0.02):
+        self.name, self.hidden_size = name, int(hidden_size)
+        self.n_heads, self.dim, self.rot_dim, self.v_dim = int(n_heads), int(dim), int(rot_dim), int(v_dim)
+        self.q_rank, self.kv_rank = int(q_rank), int(kv_rank)
+        self.scale, self.eps, self.init_std = float(scale), float(eps), init_std
+        self.window = int(window) if window else None
+        self.position = build_part("position", position)
+        if self.position.needs_apply:
+            raise ValueError(f"{name}: latent attention needs a position part that gives the kernels a rotation table")
+        self.w_down = self.w_uq = self.w_uk_t = self.w_uv = self.w_o = self.q_norm = self.kv_norm = None
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(1, self.kv_rank + self.rot_dim, self.window, self.kv_rank)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        n, H, s = self.name, self.hidden_size, ("normal", self.init_std)
+        nh, d, r, dv = self.n_heads, self.dim, self.rot_dim, self.v_dim
+        return {
+            f"{n}.dq": ParamSpec((self.q_rank, H), s), f"{n}.dq.norm": ParamSpec((self.q_rank,), ("ones",)),
+            f"{n}.uq": ParamSpec((nh * (d + r), self.q_rank), s),
+            f"{n}.dkv": ParamSpec((self.kv_rank + r, H), s), f"{n}.dkv.norm": ParamSpec((self.kv_rank,), ("ones",)),
+            f"{n}.uk": ParamSpec((nh * d, self.kv_rank), s), f"{n}.uv": ParamSpec((nh * dv, self.kv_rank), s),
+            f"{n}.o": ParamSpec((H, nh * dv), s),
+        }
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        n, nh = self.name, self.n_heads
+        self.w_down = ops.prepare_linear(concat_weights([tensors[f"{n}.dq"], tensors[f"{n}.dkv"]]))
+        self.w_uq = ops.prepare_linear(tensors[f"{n}.uq"])
+        self.w_o = ops.prepare_linear(tensors[f"{n}.o"])
+        dtype = self.w_uq.dtype
+        # per head [kv_rank, dim]: the product that moves W_uk over to the query's side
+        self.w_uk_t = tensors[f"{n}.uk"].to(dtype).view(nh, self.dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors[f"{n}.uv"].to(dtype).view(nh, self.v_dim, self.kv_rank).contiguous()
+        norms = [tensors[f"{n}.dq.norm"], tensors[f"{n}.dkv.norm"]]
+        if norms[0].dtype != norms[1].dtype:
+            norms = [w.float() for w in norms]
+        self.q_norm, self.kv_norm = norms
+
+    def forward(self, h, ctx, binding: MixerBinding):
+        cache = binding.cache
+        T, nh, t = h.shape[0], self.n_heads, ctx.timer
+        _, rot_dims, cos, sin = self.position.kernel_args(ctx)
+        slots = ctx.write_slots(cache.group) if binding.writes_cache else None
+        y = ops.linear(h, self.w_down, keep_slices=True)              # [T, q_rank + kv_rank + rot_dim]
+        cq = ops.latent_finish(y, self.q_norm, self.kv_norm, self.eps, cos, sin, rot_dims, slots, self.q_rank, self.kv_rank,
+                               self.rot_dim, cache.k, cache.v, cache.page_size, h.dtype)
+        q = ops.linear(cq, self.w_uq)                                 # [T, heads (dim + rot_dim)]
+        w_dtype = self.w_uk_t.dtype
+        qa = ops.headwise(q if q.dtype == w_dtype else q.to(w_dtype), self.w_uk_t, nh, self.dim + self.rot_dim, self.rot_dim,
+                          cos, sin, rot_dims)                         # [T, heads, kv_rank + rot_dim]
+        if t is not None:
+            t.mark("mixer.qkv")
+        a = paged_attention(qa if qa.dtype == h.dtype else qa.to(h.dtype), cache, ctx, self.window, self.scale)   # [T, heads kv_rank]
+        if t is not None:
+            t.mark("mixer.attention")
+        v = ops.headwise(a if a.dtype == w_dtype else a.to(w_dtype), self.w_uv, nh, self.kv_rank)        # [T, heads, vdim]
+        v = v.view(T, nh * self.v_dim)
+        return ops.linear(v if v.dtype == h.dtype else v.to(h.dtype), self.w_o, keep_slices=True)

@@ -1,0 +1,70 @@
+"""Mixture of experts: a router picks a few small gated feed-forwards per row and weighs their outputs.
+
+    z = W_r h (float), s = sigmoid(z) (or softmax(z) over the experts)
+    the experts lie in ``groups`` equal groups of neighbours; a group's score is the sum of its ``group_top`` highest
+    s; only experts of the ``keep_groups`` best groups can be chosen; the ``top`` highest s among them are
+    out = sum over the chosen e of w_e * W_down[e] (silu(W_gate[e] h) * (W_up[e] h)),
+    w_e = s_e, divided by the sum of the chosen s with ``renormalize``, times ``route_scale``
+
+Tensors (``<name>.``): router [experts, H], e<j>.gate and e<j>.up [ff, H], e<j>.down [H, ff]; no biases.  The experts'
+matrices are stacked at load into [experts, ff, H] and [experts, H, ff].
+
+The router and the choice run on the device, and the experts' products read each (row, choice)'s expert from device
+memory: the launches of a step depend on its layout alone, so a decode step is captured and replayed like any other.
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, register_part
+from .plan import ParamSpec
+
+
+@register_part("ffn", "moe")
+class MixtureOfExperts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, name: str, hidden_size: int, n_experts: int, top: int, ff: int, groups: int = 1, keep_groups: int = 1,
+                 group_top: int = 2, scoring: str = "sigmoid", renormalize: bool = False, route_scale: float = 1.0,
+                 init_std: float = 0.02):
+        if scoring not in ("sigmoid", "softmax"):
+            raise ValueError(f"{name}: scoring '{scoring}' unknown (sigmoid or softmax)")
+        if n_experts % groups or not 0 < keep_groups <= groups or not 0 < top <= keep_groups * (n_experts // groups):
+            raise ValueError(f"{name}: top {top} of {n_experts} experts in {groups} groups of which {keep_groups} are kept")
+        self.name, self.hidden_size = name, int(hidden_size)
+        self.n_experts, self.top, self.ff = int(n_experts), int(top), int(ff)
+        self.groups, self.keep_groups, self.group_top = int(groups), int(keep_groups), int(group_top)
+        self.scoring, self.renormalize, self.route_scale, self.init_std = scoring, bool(renormalize), float(route_scale), init_std
+        self.router = self.gate = self.up = self.down = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        n, H, s = self.name, self.hidden_size, ("normal", self.init_std)
+        out = {f"{n}.router": ParamSpec((self.n_experts, H), s)}
+        for e in range(self.n_experts):
+            out[f"{n}.e{e}.gate"] = ParamSpec((self.ff, H), s)
+            out[f"{n}.e{e}.up"] = ParamSpec((self.ff, H), s)
+            out[f"{n}.e{e}.down"] = ParamSpec((H, self.ff), s)
+        return out
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        n = self.name
+        mats = [tensors[f"{n}.e{e}.{p}"] for e in range(self.n_experts) for p in ("gate", "up", "down")] + [tensors[f"{n}.router"]]
+        dtype = mats[0].dtype if len({m.dtype for m in mats}) == 1 else torch.float32     # mixed storage is widened
+        stack = lambda p: torch.stack([tensors[f"{n}.e{e}.{p}"].to(dtype) for e in range(self.n_experts)]).contiguous()
+        self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")
+        self.router = tensors[f"{n}.router"].to(dtype).contiguous()
+
+    def route(self, h):
+        return ops.moe_route(h, self.router, self.top, self.groups, self.keep_groups, self.group_top,
+                             self.scoring == "softmax", self.renormalize, self.route_scale)
+
+    def forward(self, h, ctx):
+        x = h if h.dtype == self.router.dtype else h.to(self.router.dtype)
+        ids, weights = self.route(x)
+        if ctx.timer is not None:
+            ctx.timer.mark("ffn.route")
+        out = ops.moe_experts(x, self.gate, self.up, self.down, ids, weights)
+        return out if out.dtype == h.dtype else out.to(h.dtype)
