@@ -8,7 +8,9 @@
 // and whose value is c, with queries of kv_rank + rot_dim elements, and only c and k_r are cached.
 //
 //   ifx_latent_finish   after the down projections: RMS norm of the query latent (handed on), RMS norm of c and
-//                       rotation of k_r, both written into the paged cache (K rows [c | k_r], V columns c)
+//                       rotation of k_r, both written into the paged cache (K rows [c | k_r], V columns c; or V
+//                       columns [c | k_r] too, for attention kernels that want values as wide as keys: the sums
+//                       over k_r that they then return behind a head's kv_rank outputs are not used by anyone)
 //   ifx_headwise        out[t, h, :] = W[h] x[t, h, :] for every head (W [H][N][K]), the products by W_uk^T and
 //                       W_uv; optionally a tail of each head's input is rotated and appended to the head's output
 //                       (the rotated query part)
@@ -32,7 +34,7 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(const TY* __restrict
                                                             const float* __restrict__ cs, const float* __restrict__ sn, int rot_dims,
                                                             const int* __restrict__ slots, T* __restrict__ cq,
                                                             T* __restrict__ k_cache, T* __restrict__ v_cache, int q_rank,
-                                                            int kv_rank, int rot_dim, int page_size, float eps) {
+                                                            int kv_rank, int rot_dim, int page_size, float eps, int v_rows) {
   __shared__ float red[16];
   const size_t t = blockIdx.x;
   const int width = q_rank + kv_rank + rot_dim;
@@ -51,7 +53,7 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(const TY* __restrict
   const int slot = slots[t], page = slot / page_size, off = slot % page_size;
   const int d = kv_rank + rot_dim;
   T* krow = k_cache + (size_t)slot * d;                       // K [page][1][offset][d]
-  T* vcol = v_cache + (size_t)page * kv_rank * page_size + off;   // V [page][1][kv_rank][offset]
+  T* vcol = v_cache + (size_t)page * v_rows * page_size + off;    // V [page][1][v_rows][offset], v_rows = kv_rank or d
   const TY* yc = yr + q_rank;
   float ss = 0.f;
   for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
@@ -75,24 +77,26 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(const TY* __restrict
       v = i < half ? v * c - other * s : v * c + other * s;
     }
     krow[kv_rank + i] = from_f<T>(v);
+    if (v_rows > kv_rank) vcol[(size_t)(kv_rank + i) * page_size] = from_f<T>(v);   // values as wide as keys: see the entry point
   }
 }
 
 extern "C" int ifx_latent_finish(const void* y, int y_dtype, int n_slices, long long slice_stride, const void* wq, const void* wkv,
                                  int w_dtype, const float* cs, const float* sn, int rot_dims, const int* slots, void* cq,
                                  void* k_cache, void* v_cache, int dtype, int T, int q_rank, int kv_rank, int rot_dim,
-                                 int page_size, float eps, void* stream) {
+                                 int page_size, float eps, int v_rows, void* stream) {
   IFX_REQUIRE(T >= 0 && q_rank >= 0 && kv_rank > 0 && rot_dim >= 0, "latent_finish: bad sizes T=%d q_rank=%d kv_rank=%d rot_dim=%d", T, q_rank, kv_rank, rot_dim);
   IFX_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim, "latent_finish: %d of %d dimensions rotate", rot_dims, rot_dim);
   IFX_REQUIRE(rot_dims == 0 || (cs && sn), "latent_finish: a rotation needs its table");
   IFX_REQUIRE(!slots || (k_cache && v_cache && page_size > 0), "latent_finish: slots but no cache");
+  IFX_REQUIRE(v_rows == kv_rank || v_rows == kv_rank + rot_dim, "latent_finish: values of %d rows (the latent's %d, or %d with the key part)", v_rows, kv_rank, kv_rank + rot_dim);
   IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || y_dtype == DT_F32), "latent_finish: partial sums are float32");
   IFX_REQUIRE(w_dtype == DT_F32 || w_dtype == DT_BF16, "latent_finish: unknown weight dtype %d", w_dtype);
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
 #define LF_LAUNCH(TY, TT) \
   hipLaunchKernelGGL((latent_finish_kernel<TY, TT>), dim3(T), dim3(256), 0, s, (const TY*)y, n_slices, (size_t)slice_stride, wq, wkv, \
-                     w_dtype, cs, sn, rot_dims, slots, (TT*)cq, (TT*)k_cache, (TT*)v_cache, q_rank, kv_rank, rot_dim, page_size, eps)
+                     w_dtype, cs, sn, rot_dims, slots, (TT*)cq, (TT*)k_cache, (TT*)v_cache, q_rank, kv_rank, rot_dim, page_size, eps, v_rows)
   if (y_dtype == DT_F32 && dtype == DT_F32) LF_LAUNCH(float, float);
   else if (y_dtype == DT_F32 && dtype == DT_BF16) LF_LAUNCH(float, bf16_t);
   else if (y_dtype == DT_BF16 && dtype == DT_BF16) LF_LAUNCH(bf16_t, bf16_t);

@@ -305,7 +305,8 @@ def latent_finish(y, q_norm: Optional[torch.Tensor], kv_norm: torch.Tensor, eps:
     ``slots`` (int32 [T] = page * page_size + offset) the key/value latent under its RMS norm (``kv_norm``) and the
     key part, its first ``rot_dims`` elements turned by the table ``cos`` / ``sin`` [T, rot_dims / 2], go into the
     cache: K rows [latent | key part] (``k_cache`` [pages, 1, page_size, kv_rank + rot_dim]) and V columns
-    (``v_cache`` [pages, 1, kv_rank, page_size])."""
+    (``v_cache`` [pages, 1, kv_rank, page_size], or [pages, 1, kv_rank + rot_dim, page_size] for attention kernels that
+    want values as wide as keys: the key part is then written there as well)."""
     width = q_rank + kv_rank + rot_dim
     T = y.shape[0]
     yp, yd, n_slices, stride = _delta_args(y, (T, width), "y")
@@ -318,12 +319,15 @@ def latent_finish(y, q_norm: Optional[torch.Tensor], kv_norm: torch.Tensor, eps:
     if slots is not None:
         _check(slots, "slots", (T,), torch.int32)
         _check(k_cache, "k_cache", (None, 1, page_size, kv_rank + rot_dim), dtype)
-        _check(v_cache, "v_cache", (k_cache.shape[0], 1, kv_rank, page_size), dtype)
+        _check(v_cache, "v_cache", (k_cache.shape[0], 1, None, page_size), dtype)
+        if v_cache.shape[2] not in (kv_rank, kv_rank + rot_dim):
+            raise KernelError(f"latent_finish: values of {v_cache.shape[2]} rows (the latent's {kv_rank}, or {kv_rank + rot_dim} with the key part)")
     cq = torch.empty((T, q_rank), dtype=dtype, device=kv_norm.device) if q_rank else None
-    _call(load_module("latent"), "ifx_latent_finish", (P, I, I, LL, P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P),
+    _call(load_module("latent"), "ifx_latent_finish", (P, I, I, LL, P, P, I, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, P),
           yp, yd, n_slices, stride, _ptr(q_norm), kv_norm.data_ptr(), _dt(kv_norm), _ptr(cos) if rot_dims else 0,
           _ptr(sin) if rot_dims else 0, rot_dims, _ptr(slots), _ptr(cq), _ptr(k_cache) if slots is not None else 0,
-          _ptr(v_cache) if slots is not None else 0, _DT[dtype], T, q_rank, kv_rank, rot_dim, page_size, float(eps), _stream())
+          _ptr(v_cache) if slots is not None else 0, _DT[dtype], T, q_rank, kv_rank, rot_dim, page_size, float(eps),
+          v_cache.shape[2] if slots is not None else kv_rank, _stream())
     return cq
 
 

@@ -53,8 +53,18 @@ class LatentAttention(Mixer):
             raise ValueError(f"{name}: latent attention needs a position part that gives the kernels a rotation table")
         self.w_down = self.w_uq = self.w_uk_t = self.w_uv = self.w_o = self.q_norm = self.kv_norm = None
 
+    @property
+    def value_width(self) -> int:
+        """Width of a cached value.  The latent's, unless the matrix-core attention kernels take the key's size (they
+        are written for values as wide as keys): then the rotated key part is stored behind the latent on the value
+        side too, rot_dim / (kv_rank + rot_dim) more bytes and products on that side, and what comes back behind a
+        head's kv_rank sums is left unread."""
+        d = self.kv_rank + self.rot_dim
+        return d if (d % 16 == 0 and d <= ops.MFMA_MAX_HEAD_DIM) else self.kv_rank
+
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(1, self.kv_rank + self.rot_dim, self.window, self.kv_rank)
+        d, dv = self.kv_rank + self.rot_dim, self.value_width
+        return CacheSpec(1, d, self.window, dv if dv != d else None)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         n, H, s = self.name, self.hidden_size, ("normal", self.init_std)
@@ -95,9 +105,9 @@ class LatentAttention(Mixer):
                           cos, sin, rot_dims)                         # [T, heads, kv_rank + rot_dim]
         if t is not None:
             t.mark("mixer.qkv")
-        a = paged_attention(qa if qa.dtype == h.dtype else qa.to(h.dtype), cache, ctx, self.window, self.scale)   # [T, heads kv_rank]
+        a = paged_attention(qa if qa.dtype == h.dtype else qa.to(h.dtype), cache, ctx, self.window, self.scale)   # [T, heads value_width]
         if t is not None:
             t.mark("mixer.attention")
-        v = ops.headwise(a if a.dtype == w_dtype else a.to(w_dtype), self.w_uv, nh, self.kv_rank)        # [T, heads, vdim]
+        v = ops.headwise(a if a.dtype == w_dtype else a.to(w_dtype), self.w_uv, nh, self.value_width)    # [T, heads, vdim]
         v = v.view(T, nh * self.v_dim)
         return ops.linear(v if v.dtype == h.dtype else v.to(h.dtype), self.w_o, keep_slices=True)
