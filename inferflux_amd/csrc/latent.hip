@@ -113,6 +113,7 @@ struct HeadwiseArgs {
   const void* x; const void* w; void* out;
   const float* cs; const float* sn;
   int T, H, K, N, x_row, x_head, tail, rot_dims;
+  int tile0;      // the launch's first tile (the tail's, when only the tails are wanted)
 };
 
 #define HW_TM 16
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void headwise_kernel(HeadwiseArgs a) {
   __shared__ float xs[HW_TM][HW_TK];
   __shared__ float ws[HW_TN][HW_TK + 1];
   const int n_tiles = (a.N + HW_TN - 1) / HW_TN;
-  const int h = blockIdx.y, t0 = blockIdx.x * HW_TM, tile = blockIdx.z;
+  const int h = blockIdx.y, t0 = blockIdx.x * HW_TM, tile = blockIdx.z + a.tile0;
   const int out_head = a.N + a.tail;
   const T* x = (const T*)a.x;
   T* out = (T*)a.out;
@@ -176,15 +177,18 @@ __global__ __launch_bounds__(256) void headwise_kernel(HeadwiseArgs a) {
 }
 
 extern "C" int ifx_headwise(const void* x, const void* w, void* out, int dtype, int T, int H, int K, int N, int x_row, int x_head,
-                            int tail, const float* cs, const float* sn, int rot_dims, void* stream) {
+                            int tail, const float* cs, const float* sn, int rot_dims, int tail_only, void* stream) {
   IFX_REQUIRE(T >= 0 && H > 0 && K > 0 && N > 0 && tail >= 0, "headwise: bad sizes T=%d H=%d K=%d N=%d tail=%d", T, H, K, N, tail);
   IFX_REQUIRE(x_head >= K + tail && x_row >= (H - 1) * x_head + K + tail, "headwise: the heads do not fit the rows of x");
   IFX_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= tail, "headwise: %d of a tail of %d rotate", rot_dims, tail);
   IFX_REQUIRE(rot_dims == 0 || (cs && sn), "headwise: a rotation needs its table");
   IFX_REQUIRE(H <= 65535, "headwise: %d heads", H);
   if (T == 0) return 0;
-  HeadwiseArgs a{x, w, out, cs, sn, T, H, K, N, x_row, x_head, tail, rot_dims};
-  const dim3 grid((T + HW_TM - 1) / HW_TM, H, (N + HW_TN - 1) / HW_TN + (tail > 0 ? 1 : 0));
+  HeadwiseArgs a{x, w, out, cs, sn, T, H, K, N, x_row, x_head, tail, rot_dims, 0};
+  // tail_only: the products are somebody else's (the grouped matrix-core kernel's); only the tails are turned and copied
+  IFX_REQUIRE(!tail_only || tail > 0, "headwise: tail_only without a tail");
+  a.tile0 = tail_only ? (N + HW_TN - 1) / HW_TN : 0;
+  const dim3 grid((T + HW_TM - 1) / HW_TM, H, tail_only ? 1 : (N + HW_TN - 1) / HW_TN + (tail > 0 ? 1 : 0));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32) hipLaunchKernelGGL(headwise_kernel<float>, grid, dim3(256), 0, s, a);
   else if (dtype == DT_BF16) hipLaunchKernelGGL(headwise_kernel<bf16_t>, grid, dim3(256), 0, s, a);

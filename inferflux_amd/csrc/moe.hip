@@ -11,7 +11,7 @@
 // The two product kernels read the expert of every (row, choice) from device memory, so their grid depends on the
 // step's layout alone.  One wave forms one output element at a time (lanes across k, the fixed-order sum of
 // common.h), so a row's result does not depend on what shares its batch.  They are the path of the 32-bit mode and of
-// steps of few rows; bfloat16 steps of many rows take the grouped matrix-core product (moe_grouped.hip).
+// steps of few rows; bfloat16 steps of many rows take the grouped matrix-core product (grouped_gemm.hip).
 #include "common.h"
 
 IFX_DEFINE_LAST_ERROR()
@@ -124,7 +124,7 @@ extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, int* ids, 
 template <typename T>
 __global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ wg,
                                                                    const T* __restrict__ wu, const int* __restrict__ ids,
-                                                                   T* __restrict__ act, int K, int ff, int top) {
+                                                                   T* __restrict__ act, int K, int ff, int top, int paired) {
   const size_t item = blockIdx.x;                 // (row, choice)
   const size_t t = item / top;
   const int e = ids[item];
@@ -132,8 +132,9 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __re
   const T* x = h + t * K;
   const int i0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
   for (int i = i0; i < i0 + ROWS_PER_WAVE && i < ff; ++i) {
-    const T* g = wg + ((size_t)e * ff + i) * K;
-    const T* u = wu + ((size_t)e * ff + i) * K;
+    // paired: one tensor [E][2 ff][K] whose rows alternate 16 of Wg with the same 16 of Wu (what the grouped product reads)
+    const T* g = paired ? wg + ((size_t)e * 2 * ff + (i / 16) * 32 + i % 16) * K : wg + ((size_t)e * ff + i) * K;
+    const T* u = paired ? g + (size_t)16 * K : wu + ((size_t)e * ff + i) * K;
     float sg = 0.f, su = 0.f;
     for (int k = lane; k < K; k += WAVE) {
       const float xv = to_f(x[k]);
@@ -168,15 +169,16 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restr
 }
 
 extern "C" int ifx_moe_gate_up(const void* h, const void* wg, const void* wu, const int* ids, void* act, int dtype, int T, int K,
-                               int ff, int top, void* stream) {
+                               int ff, int top, int paired, void* stream) {
   IFX_REQUIRE(T >= 0 && K > 0 && ff > 0 && top > 0, "moe_gate_up: bad sizes T=%d K=%d ff=%d top=%d", T, K, ff, top);
+  IFX_REQUIRE(!paired || ff % 16 == 0, "moe_gate_up: paired weights need ff=%d to be a multiple of 16", ff);
   if (T == 0) return 0;
   const dim3 grid((unsigned)T * top, (ff + WAVES * ROWS_PER_WAVE - 1) / (WAVES * ROWS_PER_WAVE));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32)
-    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)h, (const float*)wg, (const float*)wu, ids, (float*)act, K, ff, top);
+    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)h, (const float*)wg, (const float*)wu, ids, (float*)act, K, ff, top, paired);
   else if (dtype == DT_BF16)
-    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)h, (const bf16_t*)wg, (const bf16_t*)wu, ids, (bf16_t*)act, K, ff, top);
+    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)h, (const bf16_t*)wg, (const bf16_t*)wu, ids, (bf16_t*)act, K, ff, top, paired);
   else IFX_FAIL("moe_gate_up: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

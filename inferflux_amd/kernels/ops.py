@@ -55,6 +55,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("layernorm", ())
     yield ("latent", ())
     yield ("moe", ())
+    yield ("grouped_gemm", ())
     yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
@@ -331,6 +332,9 @@ def latent_finish(y, q_norm: Optional[torch.Tensor], kv_norm: torch.Tensor, eps:
     return cq
 
 
+HEADWISE_GROUPED_MIN_ROWS = 32     # rows of a step from which the per-head products go to the matrix cores
+
+
 def headwise(x: torch.Tensor, weight: torch.Tensor, n_heads: int, x_head: int, tail: int = 0,
              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dims: int = 0) -> torch.Tensor:
     """A product per head: out[t, h, :N] = ``weight``[h] x[t, h] with ``weight`` [H, N, K] and head h's input the K
@@ -347,9 +351,17 @@ def headwise(x: torch.Tensor, weight: torch.Tensor, n_heads: int, x_head: int, t
         _check(cos, "cos", (T, rot_dims // 2), torch.float32)
         _check(sin, "sin", (T, rot_dims // 2), torch.float32)
     out = torch.empty((T, n_heads, N + tail), dtype=x.dtype, device=x.device)
-    _call(load_module("latent"), "ifx_headwise", (P, P, P, I, I, I, I, I, I, I, I, P, P, I, P),
+    tail_only = 0
+    if x.dtype == torch.bfloat16 and T >= HEADWISE_GROUPED_MIN_ROWS and K % 8 == 0 and x_head % 8 == 0 and x.shape[1] % 8 == 0:
+        # many rows: the products on the matrix cores, and of the other kernel only the tails
+        _call(load_module("grouped_gemm"), "ifx_headwise_grouped", (P, P, P, I, I, I, I, I, I, I, P),
+              x.data_ptr(), weight.data_ptr(), out.data_ptr(), T, n_heads, K, N, x.shape[1], x_head, N + tail, _stream())
+        if not tail:
+            return out
+        tail_only = 1
+    _call(load_module("latent"), "ifx_headwise", (P, P, P, I, I, I, I, I, I, I, I, P, P, I, I, P),
           x.data_ptr(), weight.data_ptr(), out.data_ptr(), _dt(x), T, n_heads, K, N, x.shape[1], x_head, tail,
-          _ptr(cos) if rot_dims else 0, _ptr(sin) if rot_dims else 0, rot_dims, _stream())
+          _ptr(cos) if rot_dims else 0, _ptr(sin) if rot_dims else 0, rot_dims, tail_only, _stream())
     return out
 
 
@@ -371,15 +383,28 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, groups: int = 1, 
     return ids, weights
 
 
-def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
-                     weights: torch.Tensor) -> torch.Tensor:
+def pair_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """[E, ff, K] gate and up weights (ff a multiple of 16) as one tensor [E, 2 ff, K] whose rows alternate 16 of gate with
+    the same 16 of up: a wave of the grouped product then holds a gate tile and its up tile, and the activation is its
+    epilogue."""
+    E, ff, K = gate.shape
+    if ff % 16 or up.shape != gate.shape:
+        raise KernelError(f"pair_gate_up: ff={ff} must be a multiple of 16 and both weights alike")
+    return torch.stack([gate.view(E, ff // 16, 16, K), up.view(E, ff // 16, 16, K)], dim=2).reshape(E, 2 * ff, K).contiguous()
+
+
+def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor], down: torch.Tensor, ids: torch.Tensor,
+                weights: torch.Tensor) -> torch.Tensor:
     """sum_j weights[t, j] * down[e] (silu(gate[e] h_t) * (up[e] h_t)), e = ids[t, j], row by row: every (row, choice)
-    streams its expert's weights (``gate`` / ``up`` [E, ff, K], ``down`` [E, N, ff], in h's type).  Returns [T, N]."""
+    streams its expert's weights (``gate`` / ``up`` [E, ff, K], or ``gate`` [E, 2 ff, K] from ``pair_gate_up`` and ``up``
+    None; ``down`` [E, N, ff]; all in h's type).  Returns [T, N]."""
     _check(h, "h", (None, None))
     T, K = h.shape
+    paired = up is None
     _check(gate, "gate", (None, None, K), h.dtype)
-    E, ff, _ = gate.shape
-    _check(up, "up", (E, ff, K), h.dtype)
+    E, ff = gate.shape[0], gate.shape[1] // (2 if paired else 1)
+    if not paired:
+        _check(up, "up", (E, ff, K), h.dtype)
     _check(down, "down", (E, None, ff), h.dtype)
     N = down.shape[1]
     top = ids.shape[1]
@@ -387,12 +412,55 @@ def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: tor
     _check(weights, "weights", (T, top), torch.float32)
     mod = load_module("moe")
     act = torch.empty((T, top, ff), dtype=h.dtype, device=h.device)
-    _call(mod, "ifx_moe_gate_up", (P, P, P, P, P, I, I, I, I, I, P),
-          h.data_ptr(), gate.data_ptr(), up.data_ptr(), ids.data_ptr(), act.data_ptr(), _dt(h), T, K, ff, top, _stream())
+    _call(mod, "ifx_moe_gate_up", (P, P, P, P, P, I, I, I, I, I, I, P),
+          h.data_ptr(), gate.data_ptr(), _ptr(up), ids.data_ptr(), act.data_ptr(), _dt(h), T, K, ff, top, 1 if paired else 0, _stream())
     out = torch.empty((T, N), dtype=h.dtype, device=h.device)
     _call(mod, "ifx_moe_down", (P, P, P, P, P, I, I, I, I, I, P),
           act.data_ptr(), down.data_ptr(), ids.data_ptr(), weights.data_ptr(), out.data_ptr(), _dt(h), T, N, ff, top, _stream())
     return out
+
+
+GROUPED_TILE_ITEMS = 64      # items of one expert (or rows of one head) to a workgroup of the grouped product
+
+
+def grouped_takes(dtype: torch.dtype, K: int, ff: int) -> bool:
+    """Whether the grouped matrix-core product takes experts of these sizes."""
+    return dtype == torch.bfloat16 and K % 8 == 0 and ff % 16 == 0
+
+
+def moe_experts_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
+                        weights: torch.Tensor) -> "SliceSums":
+    """The same sum for steps of many rows, on the matrix cores: the (row, choice) items are ordered by expert on the
+    device and every expert's weights meet tiles of its items (bfloat16; ``gate_up`` from ``pair_gate_up``).  Returns the
+    choices' weighted outputs as ``SliceSums`` [top, T, N] (float32), which the kernel that adds them to the stream sums
+    in the order of the choices."""
+    _check(h, "h", (None, None), torch.bfloat16)
+    T, K = h.shape
+    _check(gate_up, "gate_up", (None, None, K), torch.bfloat16)
+    E, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    _check(down, "down", (E, None, ff), torch.bfloat16)
+    N, top = down.shape[1], ids.shape[1]
+    _check(ids, "ids", (T, top), torch.int32)
+    _check(weights, "weights", (T, top), torch.float32)
+    if not grouped_takes(h.dtype, K, ff):
+        raise KernelError(f"moe_experts_grouped: K={K} must be a multiple of 8 and ff={ff} of 16")
+    mod = load_module("grouped_gemm")
+    n_items = T * top
+    max_tiles = -(-n_items // GROUPED_TILE_ITEMS) + E          # every expert may end on a tile that is not full
+    lists = torch.empty((n_items + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+    sorted_, te, ts, tc, nt = (lists[:n_items], lists[n_items:n_items + max_tiles], lists[n_items + max_tiles:n_items + 2 * max_tiles],
+                               lists[n_items + 2 * max_tiles:n_items + 3 * max_tiles], lists[n_items + 3 * max_tiles:])
+    _call(mod, "ifx_moe_sort", (P, I, I, P, P, P, P, P, P), ids.data_ptr(), n_items, E, sorted_.data_ptr(), te.data_ptr(),
+          ts.data_ptr(), tc.data_ptr(), nt.data_ptr(), _stream())
+    act = torch.empty((n_items, ff), dtype=torch.bfloat16, device=h.device)
+    _call(mod, "ifx_moe_gate_up_grouped", (P, P, P, P, P, P, P, P, I, I, I, I, P),
+          h.data_ptr(), gate_up.data_ptr(), act.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(), tc.data_ptr(),
+          nt.data_ptr(), max_tiles, K, ff, top, _stream())
+    parts = torch.empty((top, T, N), dtype=torch.float32, device=h.device)
+    _call(mod, "ifx_moe_down_grouped", (P, P, P, P, P, P, P, P, P, I, I, I, I, I, P),
+          act.data_ptr(), down.data_ptr(), parts.data_ptr(), weights.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(),
+          tc.data_ptr(), nt.data_ptr(), max_tiles, T, N, ff, top, _stream())
+    return SliceSums(parts, torch.bfloat16)
 
 
 # ----------------------------------------------------------------------------------------

@@ -23,6 +23,11 @@ from .base import FeedForward, register_part
 from .plan import ParamSpec
 
 
+# (row, choice) items of a step from which the experts' products go to the matrix cores, tiles of items of one expert
+# against that expert's weights; below, every item streams its expert's weights by itself
+GROUPED_MIN_ITEMS = 64
+
+
 @register_part("ffn", "moe")
 class MixtureOfExperts(FeedForward):
     graph_safe = True
@@ -56,6 +61,9 @@ class MixtureOfExperts(FeedForward):
         stack = lambda p: torch.stack([tensors[f"{n}.e{e}.{p}"].to(dtype) for e in range(self.n_experts)]).contiguous()
         self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")
         self.router = tensors[f"{n}.router"].to(dtype).contiguous()
+        if self.gate.is_cuda and ops.grouped_takes(dtype, self.hidden_size, self.ff):
+            # one tensor that both products read: rows of gate and up in turns of 16
+            self.gate, self.up = ops.pair_gate_up(self.gate, self.up), None
 
     def route(self, h):
         return ops.moe_route(h, self.router, self.top, self.groups, self.keep_groups, self.group_top,
@@ -66,5 +74,7 @@ class MixtureOfExperts(FeedForward):
         ids, weights = self.route(x)
         if ctx.timer is not None:
             ctx.timer.mark("ffn.route")
+        if self.up is None and x.shape[0] * self.top >= GROUPED_MIN_ITEMS:
+            return ops.moe_experts_grouped(x, self.gate, self.down, ids, weights)      # (partial sums, one per choice)
         out = ops.moe_experts(x, self.gate, self.up, self.down, ids, weights)
         return out if out.dtype == h.dtype else out.to(h.dtype)

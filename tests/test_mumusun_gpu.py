@@ -201,6 +201,54 @@ def test_experts_weighted_sum(dtype, T, K, ff, E, top):
     assert rel_err(got, want) < (1e-5 if dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("T,K,ff,E,top,N", [(200, 128, 64, 8, 2, 128), (33, 88, 48, 9, 2, 88), (700, 64, 96, 12, 4, 72), (64, 192, 16, 3, 1, 50),
+                                              (16, 40, 32, 40, 4, 40), (130, 96, 160, 5, 5, 200)])
+def test_experts_on_the_matrix_cores(T, K, ff, E, top, N):
+    """Many rows: items ordered by expert, tiles of one expert's items against its weights.  Experts nobody chose,
+    experts with several tiles, tiles that are not full; the choices come back as partial sums in choice order."""
+    h = rnd(17, T, K).bfloat16()
+    gate, up = rnd(18, E, ff, K, scale=K ** -0.5).bfloat16(), rnd(19, E, ff, K, scale=K ** -0.5).bfloat16()
+    down = rnd(20, E, N, ff, scale=ff ** -0.5).bfloat16()
+    g = torch.Generator().manual_seed(21)
+    popular = torch.randperm(E, generator=g)[:max(top, E // 2)]                  # the other experts get nothing
+    ids = torch.stack([popular[torch.randperm(popular.numel(), generator=g)[:top]] for _ in range(T)]).to(torch.int32)
+    weights = torch.rand(T, top, generator=g)
+    pairs = ops.pair_gate_up(gate.to(DEV), up.to(DEV))
+    got = ops.moe_experts_grouped(h.to(DEV), pairs, down.to(DEV), ids.to(DEV), weights.to(DEV))
+    assert tuple(got.parts.shape) == (top, T, N) and got.parts.dtype == torch.float32
+    want = torch.zeros(top, T, N, dtype=torch.float64)
+    for t in range(T):
+        for j in range(top):
+            e = int(ids[t, j])
+            want[j, t] = weights[t, j].double() * pm.expert(h[t].double(), gate[e].double(), up[e].double(), down[e].double())
+    assert rel_err(got.parts.cpu(), want) < 2e-2
+    rows = ops.moe_experts(h.to(DEV), pairs, None, down.to(DEV), ids.to(DEV), weights.to(DEV)).cpu()      # row by row from the same tensor
+    assert rel_err(rows, want.sum(0)) < 2e-2
+    stream = torch.zeros(T, N, device=DEV)                           # the kernel that takes the partial sums adds them up
+    ops.add_layernorm(stream, got, torch.ones(N, device=DEV), 1e-5, None)
+    assert rel_err(stream.cpu(), pm.layer_norm(want.sum(0), torch.ones(N, dtype=torch.float64), 1e-5)) < 2e-2
+
+
+@pytest.mark.parametrize("T,H,K,N,tail,rot", [(32, 3, 32, 96, 32, 32), (100, 6, 16, 40, 8, 4), (257, 2, 96, 24, 0, 0), (64, 1, 128, 130, 16, 16)])
+def test_headwise_product_on_the_matrix_cores(T, H, K, N, tail, rot):
+    x, w = rnd(22, T, H * (K + tail)).bfloat16(), rnd(23, H, N, K, scale=K ** -0.5).bfloat16()
+    positions = torch.arange(T, dtype=torch.int32) * 2 + 5
+    cos = sin = None
+    if rot:
+        inv = torch.tensor([30.0 ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=torch.float32, device=DEV)
+        cos, sin = ops.rope_table(positions.to(DEV), inv)
+    assert T >= ops.HEADWISE_GROUPED_MIN_ROWS
+    got = ops.headwise(x.to(DEV), w.to(DEV), H, K + tail, tail, cos, sin, rot).cpu()
+    few = torch.cat([ops.headwise(x[i:i + 8].to(DEV), w.to(DEV), H, K + tail, tail, None if cos is None else cos[i:i + 8].contiguous(),
+                                  None if sin is None else sin[i:i + 8].contiguous(), rot).cpu() for i in range(0, T, 8)])
+    xh = x.double().view(T, H, K + tail)
+    want = torch.einsum("thk,hnk->thn", xh[..., :K], w.double())
+    if tail:
+        want = torch.cat([want, pm.rotate(xh[..., K:], positions.tolist(), rot, 30.0) if rot else xh[..., K:]], dim=-1)
+    assert rel_err(got, want) < 1e-2 and rel_err(few, want) < 1e-2
+    assert torch.equal(got[..., N:], few[..., N:])
+
+
 def _paged_case(dtype, n, window, d, dv, nH, P=16, seed=20):
     """One request of n positions whose rows are all queried at once, its pages scattered over the pool; every query
     is aimed at two keys, the one on the window's inner edge and, twice as hard, the one just outside it, so that a
