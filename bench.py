@@ -50,6 +50,30 @@ WORKLOADS = {
     # steps (one graph per layout) like least
     "staggered": dict(shape=SHAPE_7B, name="Qwen2.5-7B shape", requests=64, prompt=(512, 512), new=(32, 512), chunk=512),
 }
+# Layer sizes for the comparison of the Mumusun design (attention through a latent + mixture of experts) with the dense
+# decoder at equal width, depth, vocabulary and feed-forward work per token (intermediate = top x ff): a small and a
+# medium size whose latent keys are 128 wide, which the matrix-core attention kernels take, and the medium size with
+# a key/value latent of 512 + 64, as large models of this kind have it, which goes to the plain attention kernel.
+def _mumusun_shape(width, layers, heads, dim, rot, vdim, q_rank, kv_rank, window, experts, top, ff, groups, keep, vocab=32000):
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+             "scale": (dim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}, "mask": {"size": window}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+    return {"architecture": "Mumusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
+
+
+def _dense_twin(width, layers, heads, head_dim, kv_heads, intermediate, window, vocab=32000):
+    return dict(SHAPE_7B, vocab_size=vocab, hidden_size=width, num_hidden_layers=layers, num_attention_heads=heads,
+                num_key_value_heads=kv_heads, head_dim=head_dim, intermediate_size=intermediate, max_position_embeddings=32768,
+                use_sliding_window=True, sliding_window=window, max_window_layers=0)
+
+
+DESIGN_SIZES = {
+    "small": (_mumusun_shape(1024, 8, 8, 64, 32, 64, 384, 96, 1024, 16, 2, 704, 4, 2), _dense_twin(1024, 8, 8, 128, 2, 1408, 1024)),
+    "medium": (_mumusun_shape(2048, 8, 16, 96, 32, 128, 768, 96, 2048, 64, 6, 1408, 8, 4), _dense_twin(2048, 8, 16, 128, 2, 8448, 2048)),
+    "medium-wide-latent": (_mumusun_shape(2048, 8, 16, 128, 64, 128, 1536, 512, 2048, 64, 6, 1408, 8, 4),
+                           _dense_twin(2048, 8, 16, 128, 2, 8448, 2048)),
+}
 CONTEXT = 4096
 PROMPT = 2048
 DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
@@ -73,9 +97,12 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
-    ap.add_argument("--workload", choices=["decode", "prefill", *WORKLOADS], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", *WORKLOADS], default="decode",
                     help="decode: the headline measurement; prefill: only the 2,048-token prefill, --steps times "
-                         "(for profiles); mixed3b / long14b: whole workloads through the scheduler")
+                         "(for profiles); mixed3b / long14b: whole workloads through the scheduler; mumusun: prefill and "
+                         "decode of the Mumusun design beside the dense decoder at equal size (--size, --only-design)")
+    ap.add_argument("--size", choices=["all", *DESIGN_SIZES], default="all", help="--workload mumusun: which of its sizes")
+    ap.add_argument("--only-design", choices=["both", "mumusun", "dense"], default="both", help="--workload mumusun: which of the two models")
     ap.add_argument("--no-decode-weight-copy", action="store_true",
                     help="decode from the weights' plain rows instead of the tiled copy")
     ap.add_argument("--ceilings", action=argparse.BooleanOptionalAction, default=True,
@@ -112,6 +139,8 @@ def main() -> int:
     ops.decode_weight_copy = not args.no_decode_weight_copy
     if args.workload in WORKLOADS:
         return run_workload(args, WORKLOADS[args.workload])
+    if args.workload == "mumusun":
+        return run_design_compare(args)
     shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B, "32b": SHAPE_32B,
                   "72b": SHAPE_72B}[args.shape])
     shape_name = f"Qwen2.5-{args.shape.upper()} shape"
@@ -403,6 +432,79 @@ def run_workload(args, w) -> int:
         "steps_by_tokens": {f"<={k}": n for k, n in sorted(eng.stats.step_tokens.items())},
     }
     print(json.dumps(out), flush=True)
+    return 0
+
+
+def run_design_compare(args) -> int:
+    """Prefill and decode throughput of the Mumusun design beside the dense decoder at equal size, through the step
+    function (no scheduler, no sampling): a prompt of --prompt-len tokens whole, and decode steps of 1, 8 and 64
+    requests that each hold --context tokens.  One JSON line with every number."""
+    import torch
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.engine.context import StepEntry
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+
+    tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    dev = torch.device("cuda", 0)
+    context = min(args.context, 1536)
+    results = {}
+    for size, shapes in DESIGN_SIZES.items():
+        if args.size not in ("all", size):
+            continue
+        for design, shape in zip(("mumusun", "dense"), shapes):
+            if args.only_design not in ("both", design):
+                continue
+            cfg = config_from_dict(shape)
+            model = Model(cfg).init_random(0, tdt, dev, on_host=False)
+            vocab = model.plan.vocab_size
+            gen = torch.Generator().manual_seed(3)
+            out = {}
+            batches = (1, 8, 64)
+            pages = max(batches) * (-(-(context + args.steps + args.warmup + 8) // PAGE) + 1) + -(-args.prompt_len // PAGE) + 8
+            runner = ModelRunner(model, num_pages=pages, page_size=PAGE, max_requests=max(batches) + 1)
+            # prefill
+            ids = torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
+            times = []
+            for rep in range(4):
+                runner.add_request("p")
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                runner.step([StepEntry("p", ids, [len(ids) - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                runner.free_request("p")
+            best = min(times[1:])
+            out["prefill"] = {"tokens": args.prompt_len, "ms": round(best * 1e3, 3), "tokens_per_s": round(args.prompt_len / best, 1)}
+            for b in batches:
+                rids = [f"d{i}" for i in range(b)]
+                for r in rids:
+                    runner.add_request(r)
+                    runner.step([StepEntry(r, torch.randint(0, vocab, (context,), generator=gen).tolist(), [])])
+                step = lambda: runner.step([StepEntry(r, [int(torch.randint(0, vocab, (1,), generator=gen))], [0]) for r in rids])
+                for _ in range(args.warmup + 2):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    step()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / args.steps
+                out[f"decode_b{b}"] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(b / dt, 1), "context": context}
+                for r in rids:
+                    runner.free_request(r)
+            results[f"{size}/{design}"] = out
+            note = f"[bench] {size}/{design}: prefill {out['prefill']['tokens_per_s']} tok/s, decode " + ", ".join(
+                f"b{b} {out[f'decode_b{b}']['tokens_per_s']}" for b in batches)
+            print(note, file=sys.stderr, flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prefill and decode tokens/s of the Mumusun design beside the dense decoder at equal size "
+                                f"({args.dtype}, random weights, {len(DESIGN_SIZES['small'][0]['layers'])} layers each)",
+                      "dtype": args.dtype, "data": "synthetic", "sizes": {k: {"mumusun": v[0]["layers"][0], "dense": {
+                          kk: v[1][kk] for kk in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size", "sliding_window")}}
+                          for k, v in DESIGN_SIZES.items() if args.size in ("all", k)},
+                      "results": results}), flush=True)
     return 0
 
 

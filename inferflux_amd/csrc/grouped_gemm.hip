@@ -121,23 +121,39 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a) {
   bf16x8 zero;
 #pragma unroll
   for (int i = 0; i < 8; ++i) zero[i] = (__bf16)0.f;
-  for (int k0 = 0; k0 < a.K; k0 += TK) {
-    bf16x8 wv[2], xv[2];
+  // A step's pieces are asked for one step ahead: while the matrix cores work on step s from LDS, the loads of step
+  // s + 1 are on their way into registers.
+  bf16x8 wv[2], xv[2];
+  const bf16_t* wp[2];
+  const bf16_t* xp[2];
+  int kc[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int piece = tid + 256 * p, r = piece / 8;
+    kc[p] = 8 * (piece % 8);
+    const int wrow = n0 + r, it = items[r];
+    wp[p] = wrow < a.NW ? wbase + (size_t)wrow * a.K + kc[p] : nullptr;
+    xp[p] = it >= 0 ? xbase + (size_t)(it / a.x_div) * a.x_row + kc[p] : nullptr;
+  }
+  auto fetch = [&](int k0) {
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-      const int piece = tid + 256 * p, r = piece / 8, k = k0 + 8 * (piece % 8);
-      const int wrow = n0 + r, it = items[r];
-      wv[p] = (wrow < a.NW && k < a.K) ? *(const bf16x8*)(wbase + (size_t)wrow * a.K + k) : zero;
-      xv[p] = (it >= 0 && k < a.K) ? *(const bf16x8*)(xbase + (size_t)(it / a.x_div) * a.x_row + k) : zero;
+      const bool in = k0 + kc[p] < a.K;
+      wv[p] = (wp[p] && in) ? *(const bf16x8*)(wp[p] + k0) : zero;
+      xv[p] = (xp[p] && in) ? *(const bf16x8*)(xp[p] + k0) : zero;
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < a.K; k0 += TK) {
     __syncthreads();          // everyone is done with the last step's tiles
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-      const int piece = tid + 256 * p, r = piece / 8, c = 8 * (piece % 8);
-      *(bf16x8*)&ws[r][c] = wv[p];
-      *(bf16x8*)&xs[r][c] = xv[p];
+      const int piece = tid + 256 * p, r = piece / 8;
+      *(bf16x8*)&ws[r][kc[p]] = wv[p];
+      *(bf16x8*)&xs[r][kc[p]] = xv[p];
     }
     __syncthreads();
+    if (k0 + TK < a.K) fetch(k0 + TK);
 #pragma unroll
     for (int ks = 0; ks < TK / 32; ++ks) {
       const bf16x8 bop = *(const bf16x8*)&xs[16 * wave + col][32 * ks + 8 * g4];

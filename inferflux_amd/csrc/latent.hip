@@ -176,6 +176,53 @@ __global__ __launch_bounds__(256) void headwise_kernel(HeadwiseArgs a) {
     }
 }
 
+// The same for steps of few rows: a thread owns one output element of one (row, head) and reads its weight row in
+// 16-byte pieces, all asked for at once (a wave's rows are one contiguous run of memory); no LDS, no barrier.  The sum
+// runs over k in the tiled kernel's order, so both give the same bits.
+__device__ __forceinline__ void hw_load8(const bf16_t* p, float* v) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+  const bf16x8 t = *(const bf16x8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)t[i];
+}
+__device__ __forceinline__ void hw_load8(const float* p, float* v) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void headwise_rows_kernel(HeadwiseArgs a) {
+  const int t = blockIdx.x, h = blockIdx.y, n = blockIdx.z * 256 + threadIdx.x;
+  const int out_head = a.N + a.tail;
+  const T* xt = (const T*)a.x + (size_t)t * a.x_row + (size_t)h * a.x_head;
+  T* out = (T*)a.out + ((size_t)t * a.H + h) * out_head;
+  if (n < a.N) {
+    const T* w = (const T*)a.w + ((size_t)h * a.N + n) * a.K;
+    float acc = 0.f;
+#pragma unroll 4
+    for (int k = 0; k < a.K; k += 8) {
+      float xv[8], wv[8];
+      hw_load8(xt + k, xv);
+      hw_load8(w + k, wv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc = fmaf(xv[i], wv[i], acc);
+    }
+    out[n] = from_f<T>(acc);
+  } else if (n < out_head) {
+    const int e = n - a.N, half = a.rot_dims / 2;
+    float v = to_f(xt[a.K + e]);
+    if (e < a.rot_dims) {
+      const int p = e < half ? e : e - half;
+      const float c = a.cs[(size_t)t * half + p], s = a.sn[(size_t)t * half + p];
+      const float other = to_f(xt[a.K + (e < half ? e + half : e - half)]);
+      v = e < half ? v * c - other * s : v * c + other * s;
+    }
+    out[n] = from_f<T>(v);
+  }
+}
+
+#define HW_ROWS_MAX_T 16
+
 extern "C" int ifx_headwise(const void* x, const void* w, void* out, int dtype, int T, int H, int K, int N, int x_row, int x_head,
                             int tail, const float* cs, const float* sn, int rot_dims, int tail_only, void* stream) {
   IFX_REQUIRE(T >= 0 && H > 0 && K > 0 && N > 0 && tail >= 0, "headwise: bad sizes T=%d H=%d K=%d N=%d tail=%d", T, H, K, N, tail);
@@ -188,8 +235,15 @@ extern "C" int ifx_headwise(const void* x, const void* w, void* out, int dtype, 
   // tail_only: the products are somebody else's (the grouped matrix-core kernel's); only the tails are turned and copied
   IFX_REQUIRE(!tail_only || tail > 0, "headwise: tail_only without a tail");
   a.tile0 = tail_only ? (N + HW_TN - 1) / HW_TN : 0;
-  const dim3 grid((T + HW_TM - 1) / HW_TM, H, tail_only ? 1 : (N + HW_TN - 1) / HW_TN + (tail > 0 ? 1 : 0));
   hipStream_t s = (hipStream_t)stream;
+  if (!tail_only && T <= HW_ROWS_MAX_T && K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0) {
+    const dim3 grid(T, H, (N + tail + 255) / 256);
+    if (dtype == DT_F32) hipLaunchKernelGGL(headwise_rows_kernel<float>, grid, dim3(256), 0, s, a);
+    else if (dtype == DT_BF16) hipLaunchKernelGGL(headwise_rows_kernel<bf16_t>, grid, dim3(256), 0, s, a);
+    else IFX_FAIL("headwise: unknown dtype %d", dtype);
+    IFX_LAUNCH_CHECK();
+  }
+  const dim3 grid((T + HW_TM - 1) / HW_TM, H, tail_only ? 1 : (N + HW_TN - 1) / HW_TN + (tail > 0 ? 1 : 0));
   if (dtype == DT_F32) hipLaunchKernelGGL(headwise_kernel<float>, grid, dim3(256), 0, s, a);
   else if (dtype == DT_BF16) hipLaunchKernelGGL(headwise_kernel<bf16_t>, grid, dim3(256), 0, s, a);
   else IFX_FAIL("headwise: unknown dtype %d", dtype);

@@ -19,6 +19,36 @@ IFX_DEFINE_LAST_ERROR()
 #define MAX_EXPERTS 1024
 #define MAX_TOP 32
 
+// eight consecutive elements as floats: one 16-byte load of bfloat16, two of float
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+  const bf16x8 t = *(const bf16x8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)t[i];
+}
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// R dot products of x [K] with the rows w[r] [K] at once, lanes across k in 16-byte pieces (K a multiple of 8), every
+// row's loads in flight together; each lane's partial sums, still to be added over the wave
+template <int R, typename T>
+__device__ __forceinline__ void dots8(const T* __restrict__ x, const T* const* w, int K, int lane, float* sum) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) sum[r] = 0.f;
+  for (int c = lane * 8; c < K; c += WAVE * 8) {
+    float xv[8], wv[R][8];
+    load8(x + c, xv);
+#pragma unroll
+    for (int r = 0; r < R; ++r) load8(w[r] + c, wv[r]);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sum[r] = fmaf(xv[i], wv[r][i], sum[r]);
+  }
+}
+
 struct RouteArgs {
   const void* h; const void* w; int* ids; float* weights;
   int T, K, E, top, groups, keep, group_top, softmax, renorm;
@@ -28,17 +58,33 @@ struct RouteArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(RouteArgs a) {
   __shared__ float s[MAX_EXPERTS];       // scores
-  __shared__ float gs[MAX_EXPERTS];      // group scores (-1: a group that is shut out)
+  __shared__ float gs[MAX_EXPERTS + MAX_TOP];      // group scores, and behind them the chosen scores in order
+  __shared__ int shut[MAX_EXPERTS];      // 1: a group that is shut out
   __shared__ float red[16];
   const size_t t = blockIdx.x;
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
   const T* h = (const T*)a.h + t * a.K;
   const T* w = (const T*)a.w;
-  for (int e = wid; e < a.E; e += nw) {
-    float z = 0.f;
-    for (int k = lane; k < a.K; k += WAVE) z = fmaf(to_f(h[k]), to_f(w[(size_t)e * a.K + k]), z);
-    z = wave_sum(z);
-    if (lane == 0) s[e] = z;
+  if (a.K % 8 == 0) {
+    for (int e0 = wid * 4; e0 < a.E; e0 += nw * 4) {          // four experts to a wave at a time
+      const T* rows[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) rows[r] = w + (size_t)min(e0 + r, a.E - 1) * a.K;
+      float z[4];
+      dots8<4>(h, rows, a.K, lane, z);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = wave_sum(z[r]);
+        if (lane == 0 && e0 + r < a.E) s[e0 + r] = v;
+      }
+    }
+  } else {
+    for (int e = wid; e < a.E; e += nw) {
+      float z = 0.f;
+      for (int k = lane; k < a.K; k += WAVE) z = fmaf(to_f(h[k]), to_f(w[(size_t)e * a.K + k]), z);
+      z = wave_sum(z);
+      if (lane == 0) s[e] = z;
+    }
   }
   __syncthreads();
   if (a.softmax) {
@@ -53,13 +99,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteArgs a) {
     for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] = 1.0f / (1.0f + expf(-s[e]));
   }
   __syncthreads();
-  // The choice is a few hundred comparisons: one thread makes it.
-  if (threadIdx.x != 0) return;
+  // Every thread ranks what it owns among its like (more of them score higher, or as high at a lower index): a group
+  // among the groups, then an expert among the experts of the groups that are kept.  The rank is the place in the output.
   const int per = a.E / a.groups;
-  if (a.keep < a.groups) {
-    for (int g = 0; g < a.groups; ++g) {
-      // sum of the group's group_top largest scores (scores lie in (0, 1): -1 marks one taken)
-      float sum = 0.f;
+  for (int g = threadIdx.x; g < a.groups; g += blockDim.x) {
+    float sum = 0.f;
+    if (a.keep < a.groups) {           // the sum of the group's group_top highest scores
       int taken[8];
       for (int r = 0; r < a.group_top && r < per; ++r) {
         int best = -1;
@@ -71,34 +116,32 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteArgs a) {
         taken[r] = best;
         sum += s[best];
       }
-      gs[g] = sum;
     }
-    // all but the best `keep` groups are shut out
-    for (int r = 0; r < a.groups - a.keep; ++r) {
-      int worst = -1;
-      for (int g = a.groups - 1; g >= 0; --g)          // among equals the higher index goes first
-        if (gs[g] >= 0.f && (worst < 0 || gs[g] < gs[worst])) worst = g;
-      gs[worst] = -1.f;
-    }
-  } else {
-    for (int g = 0; g < a.groups; ++g) gs[g] = 0.f;
+    gs[g] = sum;
   }
-  int chosen[MAX_TOP];
-  float total = 0.f;
-  for (int r = 0; r < a.top; ++r) {
-    int best = -1;
-    for (int e = 0; e < a.E; ++e) {
-      if (gs[e / per] < 0.f) continue;
-      bool used = false;
-      for (int q = 0; q < r; ++q) used |= chosen[q] == e;
-      if (!used && (best < 0 || s[e] > s[best])) best = e;
-    }
-    chosen[r] = best;
-    total += s[best];
+  __syncthreads();
+  for (int g = threadIdx.x; g < a.groups; g += blockDim.x) {
+    int rank = 0;
+    if (a.keep < a.groups)
+      for (int o = 0; o < a.groups; ++o) rank += (gs[o] > gs[g] || (gs[o] == gs[g] && o < g)) ? 1 : 0;
+    shut[g] = rank >= a.keep ? 1 : 0;
   }
-  for (int r = 0; r < a.top; ++r) {
-    a.ids[t * a.top + r] = chosen[r];
-    a.weights[t * a.top + r] = (a.renorm ? s[chosen[r]] / total : s[chosen[r]]) * a.scale;
+  __syncthreads();
+  for (int e = threadIdx.x; e < a.E; e += blockDim.x) {
+    if (shut[e / per]) continue;
+    int rank = 0;
+    for (int o = 0; o < a.E; ++o) rank += (!shut[o / per] && (s[o] > s[e] || (s[o] == s[e] && o < e))) ? 1 : 0;
+    if (rank < a.top) {
+      a.ids[t * a.top + rank] = e;
+      gs[a.groups + rank] = s[e];        // (gs has room behind the groups: E >= groups + top is not needed, MAX_EXPERTS + ... see below)
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < a.top) {
+    float total = 0.f;
+    for (int r = 0; r < a.top; ++r) total += gs[a.groups + r];
+    const float v = gs[a.groups + threadIdx.x];
+    a.weights[t * a.top + threadIdx.x] = (a.renorm ? v / total : v) * a.scale;
   }
 }
 
@@ -131,19 +174,38 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __re
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const T* x = h + t * K;
   const int i0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
-  for (int i = i0; i < i0 + ROWS_PER_WAVE && i < ff; ++i) {
-    // paired: one tensor [E][2 ff][K] whose rows alternate 16 of Wg with the same 16 of Wu (what the grouped product reads)
-    const T* g = paired ? wg + ((size_t)e * 2 * ff + (i / 16) * 32 + i % 16) * K : wg + ((size_t)e * ff + i) * K;
-    const T* u = paired ? g + (size_t)16 * K : wu + ((size_t)e * ff + i) * K;
-    float sg = 0.f, su = 0.f;
-    for (int k = lane; k < K; k += WAVE) {
-      const float xv = to_f(x[k]);
-      sg = fmaf(xv, to_f(g[k]), sg);
-      su = fmaf(xv, to_f(u[k]), su);
+  if (i0 >= ff) return;
+  // paired: one tensor [E][2 ff][K] whose rows alternate 16 of Wg with the same 16 of Wu (what the grouped product reads)
+  auto gate_row = [&](int i) { return paired ? wg + ((size_t)e * 2 * ff + (i / 16) * 32 + i % 16) * K : wg + ((size_t)e * ff + i) * K; };
+  auto up_row = [&](int i) { return paired ? gate_row(i) + (size_t)16 * K : wu + ((size_t)e * ff + i) * K; };
+  float sum[2 * ROWS_PER_WAVE];
+  if (K % 8 == 0) {
+    const T* rows[2 * ROWS_PER_WAVE];
+#pragma unroll
+    for (int r = 0; r < ROWS_PER_WAVE; ++r) {
+      const int i = min(i0 + r, ff - 1);
+      rows[2 * r] = gate_row(i);
+      rows[2 * r + 1] = up_row(i);
     }
-    sg = wave_sum(sg);
-    su = wave_sum(su);
-    if (lane == 0) act[item * ff + i] = from_f<T>(sg / (1.0f + expf(-sg)) * su);
+    dots8<2 * ROWS_PER_WAVE>(x, rows, K, lane, sum);
+  } else {
+    for (int r = 0; r < ROWS_PER_WAVE; ++r) {
+      const int i = min(i0 + r, ff - 1);
+      const T* g = gate_row(i);
+      const T* u = up_row(i);
+      float sg = 0.f, su = 0.f;
+      for (int k = lane; k < K; k += WAVE) {
+        const float xv = to_f(x[k]);
+        sg = fmaf(xv, to_f(g[k]), sg);
+        su = fmaf(xv, to_f(u[k]), su);
+      }
+      sum[2 * r] = sg; sum[2 * r + 1] = su;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS_PER_WAVE; ++r) {
+    const float sg = wave_sum(sum[2 * r]), su = wave_sum(sum[2 * r + 1]);
+    if (lane == 0 && i0 + r < ff) act[item * ff + i0 + r] = from_f<T>(sg / (1.0f + expf(-sg)) * su);
   }
 }
 
@@ -154,18 +216,35 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restr
   const size_t t = blockIdx.x;
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int n0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
-  for (int n = n0; n < n0 + ROWS_PER_WAVE && n < N; ++n) {
-    float y = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const int e = ids[t * top + j];
-      const T* w = wd + ((size_t)e * N + n) * ff;
-      const T* a = act + (t * top + j) * ff;
-      float s = 0.f;
-      for (int k = lane; k < ff; k += WAVE) s = fmaf(to_f(a[k]), to_f(w[k]), s);
-      y = fmaf(weights[t * top + j], wave_sum(s), y);
+  if (n0 >= N) return;
+  float y[ROWS_PER_WAVE];
+#pragma unroll
+  for (int r = 0; r < ROWS_PER_WAVE; ++r) y[r] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int e = ids[t * top + j];
+    const T* a = act + (t * top + j) * ff;
+    float sum[ROWS_PER_WAVE];
+    if (ff % 8 == 0) {
+      const T* rows[ROWS_PER_WAVE];
+#pragma unroll
+      for (int r = 0; r < ROWS_PER_WAVE; ++r) rows[r] = wd + ((size_t)e * N + min(n0 + r, N - 1)) * ff;
+      dots8<ROWS_PER_WAVE>(a, rows, ff, lane, sum);
+    } else {
+      for (int r = 0; r < ROWS_PER_WAVE; ++r) {
+        const T* w = wd + ((size_t)e * N + min(n0 + r, N - 1)) * ff;
+        float s = 0.f;
+        for (int k = lane; k < ff; k += WAVE) s = fmaf(to_f(a[k]), to_f(w[k]), s);
+        sum[r] = s;
+      }
     }
-    if (lane == 0) out[t * N + n] = from_f<T>(y);
+    const float wj = weights[t * top + j];
+#pragma unroll
+    for (int r = 0; r < ROWS_PER_WAVE; ++r) y[r] = fmaf(wj, wave_sum(sum[r]), y[r]);
   }
+  if (lane == 0)
+#pragma unroll
+    for (int r = 0; r < ROWS_PER_WAVE; ++r)
+      if (n0 + r < N) out[t * N + n0 + r] = from_f<T>(y[r]);
 }
 
 extern "C" int ifx_moe_gate_up(const void* h, const void* wg, const void* wu, const int* ids, void* act, int dtype, int T, int K,
