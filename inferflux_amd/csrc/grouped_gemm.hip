@@ -12,11 +12,12 @@
 //                      row's result does not depend on where its items lay in the order
 //   ifx_headwise_grouped      out[t][h][:N] = W[h] x[t][h], tiles of TM rows of one head
 //
-// One kernel does all three products.  A workgroup of four waves takes TM = 64 items and TN = 64 weight rows; steps of
-// 64 k-values of both are staged in LDS (16-byte pieces, rows padded by 16 bytes against bank conflicts), each wave
-// multiplies its 16 items with the four tiles of 16 weight rows: C[weight row][item], so a lane ends up with four
-// consecutive output columns of one item.  Sums run over k in ascending order whatever the tile, so an item's result
-// does not depend on what shares its tile.
+// One kernel does all three products.  A workgroup of four waves takes TM = 64 or 128 items and TN = 128 weight rows;
+// steps of 64 k-values of both are staged in LDS (16-byte pieces, rows padded by 16 bytes against bank conflicts, the
+// next step's pieces on their way into registers meanwhile).  The waves stand two by two: each multiplies 32 x MT items
+// with two tiles of 32 weight rows on the 32x32x16 matrix instruction, C[weight row][item], so a lane ends up with
+// runs of four consecutive output columns of one item.  Sums run over k in ascending order whatever the tile, so an
+// item's result does not depend on what shares its tile.
 #include "common.h"
 
 IFX_DEFINE_LAST_ERROR()
@@ -24,20 +25,20 @@ IFX_DEFINE_LAST_ERROR()
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-#define TM 64
-#define TN 64
+#define TM_MAX 128     // items to a tile: 64 or 128 (the caller's choice, the same for the list and the products)
+#define TN 128
 #define TK 64
 #define LDP (TK + 8)
 #define MAX_EXPERTS 1024
 
-extern "C" int ifx_grouped_tile_items() { return TM; }
 
 // ---------------------------------------------------------------------------------------
 // ids [n_items] -> sorted [n_items] (items of expert 0, then of expert 1, ...), tiles (expert, first place in sorted,
 // count) and their number.  One workgroup.  The order of an expert's items among themselves is not fixed; no result
 // depends on it.
-__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n_items, int E, int* __restrict__ sorted,
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n_items, int E, int TM, int* __restrict__ sorted,
                                                         int* __restrict__ tile_expert, int* __restrict__ tile_start,
                                                         int* __restrict__ tile_count, int* __restrict__ n_tiles) {
   __shared__ int cnt[MAX_EXPERTS];
@@ -69,11 +70,12 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
   }
 }
 
-extern "C" int ifx_moe_sort(const int* ids, int n_items, int E, int* sorted, int* tile_expert, int* tile_start, int* tile_count,
-                            int* n_tiles, void* stream) {
+extern "C" int ifx_moe_sort(const int* ids, int n_items, int E, int tile_items, int* sorted, int* tile_expert, int* tile_start,
+                            int* tile_count, int* n_tiles, void* stream) {
   IFX_REQUIRE(n_items >= 0 && E > 0 && E <= MAX_EXPERTS, "moe_sort: %d items, %d experts (at most %d)", n_items, E, MAX_EXPERTS);
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, n_items, E, sorted, tile_expert, tile_start,
-                     tile_count, n_tiles);
+  IFX_REQUIRE(tile_items == 64 || tile_items == 128, "moe_sort: tiles of %d items (64 or 128)", tile_items);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, n_items, E, tile_items, sorted, tile_expert,
+                     tile_start, tile_count, n_tiles);
   IFX_LAUNCH_CHECK();
 }
 
@@ -91,116 +93,128 @@ struct GroupedArgs {
   int out_head, n_groups;   // MODE_HEADS: out [T][n_groups][out_head]
 };
 
-template <int MODE>
+// MT: tiles of 32 items per wave (1: the workgroup takes 64 items, 2: 128)
+template <int MODE, int MT>
 __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a) {
+  constexpr int BM = 64 * MT;
   __shared__ __attribute__((aligned(16))) bf16_t ws[TN][LDP];
-  __shared__ __attribute__((aligned(16))) bf16_t xs[TM][LDP];
-  __shared__ int items[TM];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BM][LDP];
+  __shared__ int items[BM];
   const int tid = threadIdx.x;
   int group, start, count;
   if (MODE == MODE_HEADS) {
-    const int per = (a.T + TM - 1) / TM;
+    const int per = (a.T + BM - 1) / BM;
     group = blockIdx.x / per;
-    start = (blockIdx.x % per) * TM;
-    count = min(TM, a.T - start);
+    start = (blockIdx.x % per) * BM;
+    count = min(BM, a.T - start);
   } else {
-    if ((int)blockIdx.x >= *a.n_tiles) return;
-    group = a.tile_expert[blockIdx.x];
-    start = a.tile_start[blockIdx.x];
-    count = a.tile_count[blockIdx.x];
+    const int tile = blockIdx.x;           // (the list was cut into tiles of BM items)
+    if (tile >= *a.n_tiles) return;
+    group = a.tile_expert[tile];
+    start = a.tile_start[tile];
+    count = min(a.tile_count[tile], BM);
   }
   const int n0 = blockIdx.y * TN;
-  if (tid < TM) items[tid] = tid < count ? (MODE == MODE_HEADS ? start + tid : a.sorted[start + tid]) : -1;
+  for (int i = tid; i < BM; i += 256) items[i] = i < count ? (MODE == MODE_HEADS ? start + i : a.sorted[start + i]) : -1;
   __syncthreads();
-  const int wave = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
-  floatx4 acc[4];
+  const int wave = tid / WAVE, lane = tid % WAVE, l32 = lane & 31, hi = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;          // this wave's items: 32 MT wm ..., its weight rows: 64 wn ...
+  floatx16 acc[MT][2];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
   const bf16_t* wbase = a.w + (size_t)group * a.NW * a.K;
   const bf16_t* xbase = a.x + (size_t)group * a.x_group;
   bf16x8 zero;
 #pragma unroll
   for (int i = 0; i < 8; ++i) zero[i] = (__bf16)0.f;
   // A step's pieces are asked for one step ahead: while the matrix cores work on step s from LDS, the loads of step
-  // s + 1 are on their way into registers.
-  bf16x8 wv[2], xv[2];
-  const bf16_t* wp[2];
-  const bf16_t* xp[2];
-  int kc[2];
+  // s + 1 are on their way into registers.  Pieces of 8 k-values: 8 to a row; TN rows of W and BM rows of x.
+  constexpr int WP = TN * 8 / 256, XP = BM * 8 / 256;
+  bf16x8 wv[WP], xv[XP];
+  const bf16_t* wp[WP];
+  const bf16_t* xp[XP];
+  const int kc = 8 * (tid % 8);
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int piece = tid + 256 * p, r = piece / 8;
-    kc[p] = 8 * (piece % 8);
-    const int wrow = n0 + r, it = items[r];
-    wp[p] = wrow < a.NW ? wbase + (size_t)wrow * a.K + kc[p] : nullptr;
-    xp[p] = it >= 0 ? xbase + (size_t)(it / a.x_div) * a.x_row + kc[p] : nullptr;
+  for (int p = 0; p < WP; ++p) {
+    const int wrow = n0 + (tid + 256 * p) / 8;
+    wp[p] = wrow < a.NW ? wbase + (size_t)wrow * a.K + kc : nullptr;
+  }
+#pragma unroll
+  for (int p = 0; p < XP; ++p) {
+    const int it = items[(tid + 256 * p) / 8];
+    xp[p] = it >= 0 ? xbase + (size_t)(it / a.x_div) * a.x_row + kc : nullptr;
   }
   auto fetch = [&](int k0) {
+    const bool in = k0 + kc < a.K;
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      const bool in = k0 + kc[p] < a.K;
-      wv[p] = (wp[p] && in) ? *(const bf16x8*)(wp[p] + k0) : zero;
-      xv[p] = (xp[p] && in) ? *(const bf16x8*)(xp[p] + k0) : zero;
-    }
+    for (int p = 0; p < WP; ++p) wv[p] = (wp[p] && in) ? *(const bf16x8*)(wp[p] + k0) : zero;
+#pragma unroll
+    for (int p = 0; p < XP; ++p) xv[p] = (xp[p] && in) ? *(const bf16x8*)(xp[p] + k0) : zero;
   };
   fetch(0);
   for (int k0 = 0; k0 < a.K; k0 += TK) {
     __syncthreads();          // everyone is done with the last step's tiles
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      const int piece = tid + 256 * p, r = piece / 8;
-      *(bf16x8*)&ws[r][kc[p]] = wv[p];
-      *(bf16x8*)&xs[r][kc[p]] = xv[p];
-    }
+    for (int p = 0; p < WP; ++p) *(bf16x8*)&ws[(tid + 256 * p) / 8][kc] = wv[p];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) *(bf16x8*)&xs[(tid + 256 * p) / 8][kc] = xv[p];
     __syncthreads();
     if (k0 + TK < a.K) fetch(k0 + TK);
 #pragma unroll
-    for (int ks = 0; ks < TK / 32; ++ks) {
-      const bf16x8 bop = *(const bf16x8*)&xs[16 * wave + col][32 * ks + 8 * g4];
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      bf16x8 aop[2], bop[MT];
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const bf16x8 aop = *(const bf16x8*)&ws[16 * nt + col][32 * ks + 8 * g4];
-        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop, acc[nt], 0, 0, 0);
-      }
+      for (int nt = 0; nt < 2; ++nt) aop[nt] = *(const bf16x8*)&ws[64 * wn + 32 * nt + l32][16 * ks + 8 * hi];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) bop[mt] = *(const bf16x8*)&xs[32 * MT * wm + 32 * mt + l32][16 * ks + 8 * hi];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aop[nt], bop[mt], acc[mt][nt], 0, 0, 0);
     }
   }
-  const int m = items[16 * wave + col];
-  if (m < 0) return;
-  if (MODE == MODE_GATE_UP) {
-    // weight rows n0 .. n0 + 63 are 16 of Wg, the same 16 of Wu, the next 16 of Wg, of Wu: columns n0 / 2 .. + 31 of act
-    const int ff = a.NW / 2;
-    bf16_t* act = (bf16_t*)a.out + (size_t)m * ff;
+  // acc[mt][nt][i]: weight row n0 + 64 wn + 32 nt + 8 (i / 4) + 4 hi + i % 4 of item 32 MT wm + 32 mt + l32
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
-      const int f = n0 / 2 + 16 * pr + 4 * g4;
-      if (f >= ff) continue;
-      bf16x4 y;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = items[32 * MT * wm + 32 * mt + l32];
+    if (m < 0) continue;
+    if (MODE == MODE_GATE_UP) {
+      // a tile of 32 weight rows is 16 of Wg and the same 16 of Wu: acc[i] (i < 8) is the gate of what acc[i + 8] is the up of
+      const int ff = a.NW / 2;
+      bf16_t* act = (bf16_t*)a.out + (size_t)m * ff;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float g = acc[2 * pr][r], u = acc[2 * pr + 1][r];
-        y[r] = (__bf16)(g / (1.0f + expf(-g)) * u);
-      }
-      *(bf16x4*)(act + f) = y;
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int f = (n0 + 64 * wn + 32 * nt) / 2 + 8 * q + 4 * hi;
+          if (f >= ff) continue;
+          bf16x4 y;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float g = acc[mt][nt][4 * q + r], u = acc[mt][nt][8 + 4 * q + r];
+            y[r] = (__bf16)(g / (1.0f + expf(-g)) * u);
+          }
+          *(bf16x4*)(act + f) = y;
+        }
+    } else {
+      const float wgt = MODE == MODE_DOWN ? a.weights[m] : 1.f;
+      float* of = MODE == MODE_DOWN ? (float*)a.out + ((size_t)(m % a.top) * a.T + m / a.top) * a.NW : nullptr;
+      bf16_t* ob = MODE == MODE_HEADS ? (bf16_t*)a.out + ((size_t)m * a.n_groups + group) * a.out_head : nullptr;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int n = n0 + 64 * wn + 32 * nt + 8 * (i / 4) + 4 * hi + i % 4;
+          if (n >= a.NW) continue;
+          if (MODE == MODE_DOWN) of[n] = wgt * acc[mt][nt][i];
+          else ob[n] = (bf16_t)acc[mt][nt][i];
+        }
     }
-  } else if (MODE == MODE_DOWN) {
-    const float wgt = a.weights[m];
-    float* o = (float*)a.out + ((size_t)(m % a.top) * a.T + m / a.top) * a.NW;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n0 + 16 * nt + 4 * g4 + r;
-        if (n < a.NW) o[n] = wgt * acc[nt][r];
-      }
-  } else {
-    bf16_t* o = (bf16_t*)a.out + ((size_t)m * a.n_groups + group) * a.out_head;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n0 + 16 * nt + 4 * g4 + r;
-        if (n < a.NW) o[n] = (bf16_t)acc[nt][r];
-      }
   }
 }
 
@@ -210,25 +224,31 @@ static int check_common(int K, int x_row, int x_group) {
 
 // act [n_items][ff] (bfloat16) from x [T][K] and the paired weights w [E][2 ff][K]; item i is row i / top.
 extern "C" int ifx_moe_gate_up_grouped(const void* x, const void* w, void* act, const int* sorted, const int* tile_expert,
-                                       const int* tile_start, const int* tile_count, const int* n_tiles, int max_tiles, int K,
-                                       int ff, int top, void* stream) {
+                                       const int* tile_start, const int* tile_count, const int* n_tiles, int max_tiles, int tile_items,
+                                       int K, int ff, int top, void* stream) {
   IFX_REQUIRE(check_common(K, K, 0) && ff > 0 && ff % 16 == 0 && top > 0, "moe_gate_up_grouped: K=%d must be a multiple of 8, ff=%d of 16", K, ff);
   if (max_tiles <= 0) return 0;
   GroupedArgs a{(const bf16_t*)x, (const bf16_t*)w, act, sorted, tile_expert, tile_start, tile_count, n_tiles, nullptr,
                 K, 2 * ff, top, K, 0, 0, top, 0, 0};
-  hipLaunchKernelGGL(grouped_kernel<MODE_GATE_UP>, dim3(max_tiles, (2 * ff + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
+  const dim3 grid(max_tiles, (2 * ff + TN - 1) / TN);
+  if (tile_items == 128) hipLaunchKernelGGL((grouped_kernel<MODE_GATE_UP, 2>), grid, dim3(256), 0, (hipStream_t)stream, a);
+  else if (tile_items == 64) hipLaunchKernelGGL((grouped_kernel<MODE_GATE_UP, 1>), grid, dim3(256), 0, (hipStream_t)stream, a);
+  else IFX_FAIL("moe_gate_up_grouped: tiles of %d items (64 or 128)", tile_items);
   IFX_LAUNCH_CHECK();
 }
 
 // parts [top][T][N] (float) = weights[item] * (Wd[e] act[item]), w [E][N][ff]
 extern "C" int ifx_moe_down_grouped(const void* act, const void* w, float* parts, const float* weights, const int* sorted,
                                     const int* tile_expert, const int* tile_start, const int* tile_count, const int* n_tiles,
-                                    int max_tiles, int T, int N, int ff, int top, void* stream) {
+                                    int max_tiles, int tile_items, int T, int N, int ff, int top, void* stream) {
   IFX_REQUIRE(check_common(ff, ff, 0) && N > 0 && top > 0 && T >= 0, "moe_down_grouped: ff=%d must be a multiple of 8", ff);
   if (max_tiles <= 0 || T == 0) return 0;
   GroupedArgs a{(const bf16_t*)act, (const bf16_t*)w, parts, sorted, tile_expert, tile_start, tile_count, n_tiles, weights,
                 ff, N, 1, ff, 0, T, top, 0, 0};
-  hipLaunchKernelGGL(grouped_kernel<MODE_DOWN>, dim3(max_tiles, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
+  const dim3 grid(max_tiles, (N + TN - 1) / TN);
+  if (tile_items == 128) hipLaunchKernelGGL((grouped_kernel<MODE_DOWN, 2>), grid, dim3(256), 0, (hipStream_t)stream, a);
+  else if (tile_items == 64) hipLaunchKernelGGL((grouped_kernel<MODE_DOWN, 1>), grid, dim3(256), 0, (hipStream_t)stream, a);
+  else IFX_FAIL("moe_down_grouped: tiles of %d items (64 or 128)", tile_items);
   IFX_LAUNCH_CHECK();
 }
 
@@ -239,6 +259,7 @@ extern "C" int ifx_headwise_grouped(const void* x, const void* w, void* out, int
   if (T <= 0) return 0;
   GroupedArgs a{(const bf16_t*)x, (const bf16_t*)w, out, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                 K, N, 1, x_row, x_head, T, 1, out_head, H};
-  hipLaunchKernelGGL(grouped_kernel<MODE_HEADS>, dim3(((T + TM - 1) / TM) * H, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
+  if (T > 64) hipLaunchKernelGGL((grouped_kernel<MODE_HEADS, 2>), dim3(((T + 127) / 128) * H, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL((grouped_kernel<MODE_HEADS, 1>), dim3(((T + 63) / 64) * H, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
   IFX_LAUNCH_CHECK();
 }

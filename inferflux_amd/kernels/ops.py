@@ -420,7 +420,10 @@ def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor],
     return out
 
 
-GROUPED_TILE_ITEMS = 64      # items of one expert (or rows of one head) to a workgroup of the grouped product
+def grouped_tile_items(n_items: int, n_experts: int) -> int:
+    """Items of one expert to a workgroup of the grouped product: 128 where the experts get that many on average (every
+    weight tile fetched then serves twice the items), else 64 (steps of few rows, whose tiles are mostly empty)."""
+    return 128 if n_items >= 128 * n_experts else 64
 
 
 def grouped_takes(dtype: torch.dtype, K: int, ff: int) -> bool:
@@ -446,20 +449,21 @@ def moe_experts_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
         raise KernelError(f"moe_experts_grouped: K={K} must be a multiple of 8 and ff={ff} of 16")
     mod = load_module("grouped_gemm")
     n_items = T * top
-    max_tiles = -(-n_items // GROUPED_TILE_ITEMS) + E          # every expert may end on a tile that is not full
+    tile_items = grouped_tile_items(n_items, E)
+    max_tiles = -(-n_items // tile_items) + E          # every expert may end on a tile that is not full
     lists = torch.empty((n_items + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
     sorted_, te, ts, tc, nt = (lists[:n_items], lists[n_items:n_items + max_tiles], lists[n_items + max_tiles:n_items + 2 * max_tiles],
                                lists[n_items + 2 * max_tiles:n_items + 3 * max_tiles], lists[n_items + 3 * max_tiles:])
-    _call(mod, "ifx_moe_sort", (P, I, I, P, P, P, P, P, P), ids.data_ptr(), n_items, E, sorted_.data_ptr(), te.data_ptr(),
+    _call(mod, "ifx_moe_sort", (P, I, I, I, P, P, P, P, P, P), ids.data_ptr(), n_items, E, tile_items, sorted_.data_ptr(), te.data_ptr(),
           ts.data_ptr(), tc.data_ptr(), nt.data_ptr(), _stream())
     act = torch.empty((n_items, ff), dtype=torch.bfloat16, device=h.device)
-    _call(mod, "ifx_moe_gate_up_grouped", (P, P, P, P, P, P, P, P, I, I, I, I, P),
+    _call(mod, "ifx_moe_gate_up_grouped", (P, P, P, P, P, P, P, P, I, I, I, I, I, P),
           h.data_ptr(), gate_up.data_ptr(), act.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(), tc.data_ptr(),
-          nt.data_ptr(), max_tiles, K, ff, top, _stream())
+          nt.data_ptr(), max_tiles, tile_items, K, ff, top, _stream())
     parts = torch.empty((top, T, N), dtype=torch.float32, device=h.device)
-    _call(mod, "ifx_moe_down_grouped", (P, P, P, P, P, P, P, P, P, I, I, I, I, I, P),
+    _call(mod, "ifx_moe_down_grouped", (P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P),
           act.data_ptr(), down.data_ptr(), parts.data_ptr(), weights.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(),
-          tc.data_ptr(), nt.data_ptr(), max_tiles, T, N, ff, top, _stream())
+          tc.data_ptr(), nt.data_ptr(), max_tiles, tile_items, T, N, ff, top, _stream())
     return SliceSums(parts, torch.bfloat16)
 
 
