@@ -37,15 +37,28 @@ template <int R, typename T>
 __device__ __forceinline__ void dots8(const T* __restrict__ x, const T* const* w, int K, int lane, float* sum) {
 #pragma unroll
   for (int r = 0; r < R; ++r) sum[r] = 0.f;
-  for (int c = lane * 8; c < K; c += WAVE * 8) {
-    float xv[8], wv[R][8];
-    load8(x + c, xv);
+  // two pieces of every row a trip: 2 (R + 1) loads of 16 bytes in flight per lane
+  for (int c = lane * 8; c < K; c += 2 * WAVE * 8) {
+    const int c2 = c + WAVE * 8;
+    const bool more = c2 < K;
+    float xv[2][8], wv[2][R][8];
+    load8(x + c, xv[0]);
 #pragma unroll
-    for (int r = 0; r < R; ++r) load8(w[r] + c, wv[r]);
+    for (int r = 0; r < R; ++r) load8(w[r] + c, wv[0][r]);
+    if (more) {
+      load8(x + c2, xv[1]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) load8(w[r] + c2, wv[1][r]);
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sum[r] = fmaf(xv[i], wv[r][i], sum[r]);
+      for (int i = 0; i < 8; ++i) sum[r] = fmaf(xv[0][i], wv[0][r][i], sum[r]);
+    if (more)
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum[r] = fmaf(xv[1][i], wv[1][r][i], sum[r]);
   }
 }
 
@@ -56,7 +69,7 @@ struct RouteArgs {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(RouteArgs a) {
+__global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
   __shared__ float s[MAX_EXPERTS];       // scores
   __shared__ float gs[MAX_EXPERTS + MAX_TOP];      // group scores, and behind them the chosen scores in order
   __shared__ int shut[MAX_EXPERTS];      // 1: a group that is shut out
@@ -153,9 +166,11 @@ extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, int* ids, 
   IFX_REQUIRE(top > 0 && top <= MAX_TOP && top <= keep * (E / groups), "moe_route: top %d of %d x %d experts", top, keep, E / groups);
   if (T == 0) return 0;
   RouteArgs a{h, w, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale};
+  // a wave takes four experts at a time: as many waves as that takes, up to 16 (the scores are a chain of trips to memory otherwise)
+  const int threads = WAVE * (E <= 16 ? 4 : (E <= 32 ? 8 : 16));
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(256), 0, s, a);
-  else if (dtype == DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(256), 0, s, a);
+  if (dtype == DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(threads), 0, s, a);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(threads), 0, s, a);
   else IFX_FAIL("moe_route: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

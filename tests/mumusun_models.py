@@ -41,6 +41,11 @@ CONFIGS = {
         _layer(_mixer(4, 32, 16, 32, 64, 48, 0.144, 10000.0, window=48), _moe(8, 2, 64, 2, 1)),
         _layer(_mixer(4, 32, 16, 32, 64, 48, 0.144, 10000.0), _moe(8, 2, 64, 4, 3)),
     ]},
+    # nothing a multiple of 8: every product takes its general path (the vector loads and matrix-core tiles do not apply)
+    "S": {"architecture": "Mumusun", "vocab": 99, "width": 100, "norm": {"eps": 1e-5}, "layers": [
+        _layer(_mixer(3, 10, 6, 14, 30, 27, 0.25, 3000.0, dims=6, window=19), _moe(5, 2, 50)),
+        _layer(_mixer(2, 18, 2, 9, 21, 35, 0.22, 100.0, window=1000), _moe(6, 3, 22, 3, 2)),
+    ]},
 }
 
 

@@ -143,3 +143,19 @@ def test_plain_model_is_causal_and_windowed(tmp_path):
     streams = []
     pm.forward(cfg, W, ids[:9], streams)
     assert len(streams) == 2 and streams[0].shape == (9, 88)
+
+
+def test_command_line_writes_and_inspects_a_model(tmp_path, capsys):
+    import json
+    from inferflux_amd import cli
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(mm.config("Q")))
+    out = str(tmp_path / "model")
+    assert cli.main(["random-weights", "--config", str(cfg_file), "--out", out, "--seed", "3"]) == 0
+    capsys.readouterr()
+    assert cli.main(["inspect", "--model", out]) == 0
+    report = json.loads(capsys.readouterr().out)
+    assert report["missing"] == [] and report["unexpected"] == [] and report["tensors_expected"] == report["tensors_in_file"]
+    assert report["config"]["architecture"] == "Mumusun" and report["config"]["layers"][1]["mixer"]["rot"]["dims"] == 4
+    cfg, W = pm.load_folder(out)                      # the plain implementation reads what the package wrote
+    assert pm.forward(cfg, W, [1, 2, 3]).shape == (3, 131)

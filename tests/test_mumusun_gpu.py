@@ -406,7 +406,7 @@ def test_long_decoding_gives_pages_back_as_the_windows_pass(dtype, folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_replay_of_traces_with_pages_and_slots_used_again(name, dtype, folders, tmp_path):
     """Through bin/trace_run as a user would: whole, prefill then decode, portions, and mixed steps of up to four live
     requests, one process, a pool so small that pages and slots are used again."""
@@ -460,3 +460,15 @@ def test_greedy_generation_through_the_engine(name, folders):
         for i, tok in enumerate(o.token_ids):
             row = full[len(p) - 1 + i]
             assert row[tok] >= row.max() - 0.06 * row.abs().max(), (name, i)
+
+
+def test_completion_from_the_command_line(folders, capsys):
+    from inferflux_amd import cli
+    folder = folders["Q", "float32"]
+    cfg, W = pm.load_folder(folder)
+    prompt = ids_of(90, 21, 131)
+    assert cli.main(["completion", "--model", folder, "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "7", "--temperature", "0",
+                     "--ignore-eos", "--dtype", "float32", "--kv-pages", "32", "--max-parallel-sequences", "2"]) == 0
+    said = capsys.readouterr().out
+    want = pm.greedy_generate(cfg, W, prompt, 7)
+    assert str(want)[1:-1].replace(" ", "") in said.replace(" ", ""), (want, said)
