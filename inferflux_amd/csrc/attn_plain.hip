@@ -21,6 +21,18 @@ IFX_DEFINE_LAST_ERROR()
 #define DC (MAX_D / WAVE)
 #define WAVES_PER_BLOCK 4
 
+// eight consecutive elements as floats: one 16-byte load of bfloat16, two of float
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+  const bf16x8 t = *(const bf16x8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)t[i];
+}
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 struct AttnArgs {
   const void* q;
   const void* k_cache;
@@ -72,7 +84,16 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
       off = j % P;
       const T* kr = Kc + (((size_t)page * a.nKV + kvh) * P + off) * d;
       float dot = 0.f;
-      for (int e = 0; e < d; ++e) dot = fmaf(q_s[wid][e], to_f(kr[e]), dot);
+      if (d % 8 == 0) {        // the key's row in 16-byte pieces; the same additions in the same order
+        for (int e = 0; e < d; e += 8) {
+          float kv[8];
+          load8(kr + e, kv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dot = fmaf(q_s[wid][e + i], kv[i], dot);
+        }
+      } else {
+        for (int e = 0; e < d; ++e) dot = fmaf(q_s[wid][e], to_f(kr[e]), dot);
+      }
       s = dot * a.scale;
     }
     const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds key `lo` or later, up to pos
@@ -81,6 +102,29 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
     l = l * alpha + wave_sum(p);
 #pragma unroll
     for (int c = 0; c < DC; ++c) acc[c] *= alpha;
+    if (P % 8 == 0) {
+      // Eight keys at a time: they lie in one page, where a value element's eight entries are 16 consecutive bytes.
+      // Keys outside the range have weight 0 and their entries (stale or zero, never written with anything that is
+      // not finite) add nothing; an element's sum still runs over the keys in ascending order.
+      for (int g = 0; g < WAVE; g += 8) {
+        const int j0 = t0 + g;
+        if (j0 > pos || j0 + 7 < lo) continue;                  // uniform over the wave
+        float pj[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pj[i] = __shfl(p, g + i, WAVE);
+        const T* vb = Vc + ((size_t)table[j0 / P] * a.nKV + kvh) * dv * P + j0 % P;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          const int e = lane + c * WAVE;
+          if (e < dv) {
+            float vv[8];
+            load8(vb + (size_t)e * P, vv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[c] = fmaf(pj[i], vv[i], acc[c]);
+          }
+        }
+      }
+    } else
     for (int jj = 0; jj < WAVE; ++jj) {
       const float pj = __shfl(p, jj, WAVE);
       const int pg = __shfl(page, jj, WAVE), of = __shfl(off, jj, WAVE);
