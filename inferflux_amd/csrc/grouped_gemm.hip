@@ -205,14 +205,31 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a) {
       const float wgt = MODE == MODE_DOWN ? a.weights[m] : 1.f;
       float* of = MODE == MODE_DOWN ? (float*)a.out + ((size_t)(m % a.top) * a.T + m / a.top) * a.NW : nullptr;
       bf16_t* ob = MODE == MODE_HEADS ? (bf16_t*)a.out + ((size_t)m * a.n_groups + group) * a.out_head : nullptr;
+      const bool whole4 = a.NW % 4 == 0 && (MODE == MODE_DOWN || a.out_head % 4 == 0);      // runs of four columns, stored at once
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int n = n0 + 64 * wn + 32 * nt + 8 * (i / 4) + 4 * hi + i % 4;
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + 64 * wn + 32 * nt + 8 * q + 4 * hi;
           if (n >= a.NW) continue;
-          if (MODE == MODE_DOWN) of[n] = wgt * acc[mt][nt][i];
-          else ob[n] = (bf16_t)acc[mt][nt][i];
+          if (whole4) {
+            if (MODE == MODE_DOWN) {
+              *(floatx4*)(of + n) = floatx4{wgt * acc[mt][nt][4 * q], wgt * acc[mt][nt][4 * q + 1], wgt * acc[mt][nt][4 * q + 2],
+                                            wgt * acc[mt][nt][4 * q + 3]};
+            } else {
+              bf16x4 y;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) y[r] = (__bf16)acc[mt][nt][4 * q + r];
+              *(bf16x4*)(ob + n) = y;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              if (n + r >= a.NW) continue;
+              if (MODE == MODE_DOWN) of[n + r] = wgt * acc[mt][nt][4 * q + r];
+              else ob[n + r] = (bf16_t)acc[mt][nt][4 * q + r];
+            }
+          }
         }
     }
   }

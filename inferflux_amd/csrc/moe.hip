@@ -1,6 +1,7 @@
 // Mixture of experts: the router and the experts' products for rows that each choose their own experts.
 //
-//   ifx_moe_route     z = W_r h in float, score s = sigmoid(z) (or softmax over the experts), choice of `top` experts
+//   ifx_moe_route     z = W_r h in float (formed here for steps of few rows, else given: a product of many rows belongs
+//                     to the product kernels), score s = sigmoid(z) (or softmax over the experts), choice of `top` experts
 //                     among those of the best `keep` of `groups` equal groups of neighbouring experts (a group's
 //                     score: the sum of its `group_top` largest scores); the weights are the chosen scores as they
 //                     are or divided by their sum.  Writes ids [T][top] (int32) and weights [T][top] (float), in
@@ -63,7 +64,7 @@ __device__ __forceinline__ void dots8(const T* __restrict__ x, const T* const* w
 }
 
 struct RouteArgs {
-  const void* h; const void* w; int* ids; float* weights;
+  const void* h; const void* w; const float* z; int* ids; float* weights;
   int T, K, E, top, groups, keep, group_top, softmax, renorm;
   float scale;
 };
@@ -78,7 +79,9 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
   const T* h = (const T*)a.h + t * a.K;
   const T* w = (const T*)a.w;
-  if (a.K % 8 == 0) {
+  if (a.z) {                     // the logits are somebody else's product (steps of many rows)
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] = a.z[t * a.E + e];
+  } else if (a.K % 8 == 0) {
     for (int e0 = wid * 4; e0 < a.E; e0 += nw * 4) {          // four experts to a wave at a time
       const T* rows[4];
 #pragma unroll
@@ -158,18 +161,19 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
   }
 }
 
-extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, int* ids, float* weights, int T, int K, int E, int top,
-                             int groups, int keep, int group_top, int softmax, int renorm, float scale, void* stream) {
+extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, const float* z, int* ids, float* weights, int T, int K, int E,
+                             int top, int groups, int keep, int group_top, int softmax, int renorm, float scale, void* stream) {
+  IFX_REQUIRE(z || (h && w), "moe_route: neither logits nor the rows and the router's weight");
   IFX_REQUIRE(T >= 0 && K > 0 && E > 0 && E <= MAX_EXPERTS, "moe_route: %d experts (at most %d), K=%d", E, MAX_EXPERTS, K);
   IFX_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups, "moe_route: %d experts in %d groups of which %d are kept", E, groups, keep);
   IFX_REQUIRE(group_top > 0 && group_top <= 8, "moe_route: a group's score sums its %d largest (1-8)", group_top);
   IFX_REQUIRE(top > 0 && top <= MAX_TOP && top <= keep * (E / groups), "moe_route: top %d of %d x %d experts", top, keep, E / groups);
   if (T == 0) return 0;
-  RouteArgs a{h, w, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale};
+  RouteArgs a{h, w, z, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale};
   // a wave takes four experts at a time: as many waves as that takes, up to 16 (the scores are a chain of trips to memory otherwise)
-  const int threads = WAVE * (E <= 16 ? 4 : (E <= 32 ? 8 : 16));
+  const int threads = z ? WAVE * (E <= 64 ? 1 : 4) : WAVE * (E <= 16 ? 4 : (E <= 32 ? 8 : 16));
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(threads), 0, s, a);
+  if (z || dtype == DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(threads), 0, s, a);
   else if (dtype == DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(threads), 0, s, a);
   else IFX_FAIL("moe_route: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();

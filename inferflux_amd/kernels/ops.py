@@ -365,20 +365,28 @@ def headwise(x: torch.Tensor, weight: torch.Tensor, n_heads: int, x_head: int, t
     return out
 
 
-def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, groups: int = 1, keep_groups: int = 1, group_top: int = 2,
+ROUTE_FUSED_MAX_ROWS = 16       # rows up to which the router's kernel forms the logits itself
+
+
+def moe_route(h: torch.Tensor, router, top: int, groups: int = 1, keep_groups: int = 1, group_top: int = 2,
               softmax: bool = False, renormalize: bool = False, scale: float = 1.0):
-    """The router of a mixture of experts, in float: scores of ``router`` [E, K] times the rows of ``h`` [T, K] through a
-    sigmoid (or a softmax over the experts), the ``top`` highest among the experts of the best ``keep_groups`` of
-    ``groups`` equal groups of neighbours (a group scores the sum of its ``group_top`` highest).  Returns (ids int32
-    [T, top], weights float32 [T, top]): the chosen scores, divided by their sum with ``renormalize``, times ``scale``."""
+    """The router of a mixture of experts, in float: scores of ``router`` [E, K] (a tensor or a ``LinearWeight``) times the
+    rows of ``h`` [T, K] through a sigmoid (or a softmax over the experts), the ``top`` highest among the experts of the best
+    ``keep_groups`` of ``groups`` equal groups of neighbours (a group scores the sum of its ``group_top`` highest).  Returns
+    (ids int32 [T, top], weights float32 [T, top]): the chosen scores, divided by their sum with ``renormalize``, times
+    ``scale``.  Up to ``ROUTE_FUSED_MAX_ROWS`` rows the kernel forms the logits itself; more rows in bfloat16 get them from
+    ``linear`` with float32 sums and output."""
     _check(h, "h", (None, None))
     T, K = h.shape
-    _check(router, "router", (None, K), h.dtype)
-    E = router.shape[0]
+    rows = router.rows if isinstance(router, LinearWeight) else router
+    _check(rows, "router", (None, K), h.dtype)
+    E = rows.shape[0]
+    # (in 32-bit the kernel forms them whatever the rows: a row's sums then never depend on what shares its step)
+    z = linear(h, router, out_dtype=torch.float32) if (T > ROUTE_FUSED_MAX_ROWS and h.dtype == torch.bfloat16) else None
     ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
-    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, I, I, I, I, I, I, I, I, I, F, P),
-          h.data_ptr(), router.data_ptr(), _dt(h), ids.data_ptr(), weights.data_ptr(), T, K, E, top, groups, keep_groups,
+    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P),
+          h.data_ptr(), rows.data_ptr(), _dt(h), _ptr(z), ids.data_ptr(), weights.data_ptr(), T, K, E, top, groups, keep_groups,
           group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _stream())
     return ids, weights
 

@@ -60,7 +60,7 @@ class MixtureOfExperts(FeedForward):
         dtype = mats[0].dtype if len({m.dtype for m in mats}) == 1 else torch.float32     # mixed storage is widened
         stack = lambda p: torch.stack([tensors[f"{n}.e{e}.{p}"].to(dtype) for e in range(self.n_experts)]).contiguous()
         self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")
-        self.router = tensors[f"{n}.router"].to(dtype).contiguous()
+        self.router = ops.prepare_linear(tensors[f"{n}.router"].to(dtype).contiguous())     # (steps of many rows take its product from ``linear``)
         if self.gate.is_cuda and ops.grouped_takes(dtype, self.hidden_size, self.ff):
             # one tensor that both products read: rows of gate and up in turns of 16
             self.gate, self.up = ops.pair_gate_up(self.gate, self.up), None
