@@ -65,12 +65,35 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
                                                             TC* __restrict__ cast_out, int H, float eps) {
   extern __shared__ float row[];
   __shared__ float red[16];
+  constexpr int NV = 8;          // rows of up to 256 NV columns: the stream and the weight are asked for before the sums
   const size_t t = blockIdx.x;
+  float* s = stream + t * H;
+  const bool ahead = H <= 256 * NV;
+  float sv[NV], wv[NV];
+  if (ahead) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int i = threadIdx.x + 256 * v;
+      sv[v] = i < H ? s[i] : 0.f;
+      wv[v] = i < H ? load_dyn(weight, w_dtype, i) : 0.f;
+    }
+  }
   for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = sliced(delta + t * H, i, n_slices, slice_stride);
   __syncthreads();
   float mean, rstd;
   moments(row, H, eps, red, mean, rstd);
-  float* s = stream + t * H;
+  if (ahead) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int i = threadIdx.x + 256 * v;
+      if (i < H) {
+        const float x = sv[v] + (row[i] - mean) * rstd * wv[v];
+        s[i] = x;
+        if (cast_out) cast_out[t * H + i] = from_f<TC>(x);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     const float v = s[i] + (row[i] - mean) * rstd * load_dyn(weight, w_dtype, i);
     s[i] = v;

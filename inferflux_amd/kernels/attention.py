@@ -2,7 +2,7 @@
 
 Every choice computes the same function (causal, optionally windowed, grouped-query attention
 over the paged cache); they differ in speed and in which sizes they accept.  In bfloat16 with a
-head size the matrix-core module takes, requests that bring at least TILE_MIN rows go to the
+head size the matrix-core module takes (up to 128, values as wide as keys), requests that bring at least TILE_MIN rows go to the
 tile kernel (tiles of as many rows as the compiled module says; keys in splits when the tiles are
 few and their pasts long) and all other rows (decode tokens, short portions) to the row kernel;
 everything else (float32, other head sizes) goes to the plain kernel.
@@ -227,7 +227,12 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     """q [T, nH, d] of this step's rows against ``cache`` (a LayerCache); returns [T, nH*d]."""
     T, nH, d = q.shape
     table = ctx.block_table(cache.group)
-    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:    # (values of another width: the plain kernel)
+    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
+        # values of another width than the keys, or heads wider than a wave's registers hold: one shared kv head (attention
+        # through a latent) has a matrix-core kernel of its own, everything else (32-bit, odd sizes) the plain kernel
+        if ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
+            chunk, splits = ops.wide_launch_shape(T, nH, ctx.kv_bound)
+            return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits)
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
     # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.

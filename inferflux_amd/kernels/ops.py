@@ -60,6 +60,8 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
             yield _tile_module(d, qt)[:2]
+    for dk, dv in WIDE_DIMS_PREBUILT:
+        yield ("attn_wide", (("K_DIM", dk), ("V_DIM", dv)))
 
 
 def _tile_module(head_dim: int, qt: int):
@@ -1011,6 +1013,55 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, dv, page_size,
           int(window or 0), float(scale), _stream())
+    return out
+
+
+WIDE_MAX_K_DIM, WIDE_MAX_V_DIM = 1024, 512
+WIDE_DIMS_PREBUILT = ((576, 512),)      # compiled ahead by build_all(); any other pair of widths when a model first needs it
+
+
+def wide_attention_supported(dtype: torch.dtype, n_kv_heads: int, k_dim: int, v_dim: int, page_size: int) -> bool:
+    """Whether ``attention_wide`` takes this cache: bfloat16, one kv head that all query heads share, keys of a multiple
+    of 8 and values of a multiple of 16 elements, pages of a power of two from 16."""
+    return (dtype == torch.bfloat16 and n_kv_heads == 1 and k_dim % 8 == 0 and 0 < k_dim <= WIDE_MAX_K_DIM and v_dim % 16 == 0
+            and 0 < v_dim <= WIDE_MAX_V_DIM and page_size >= 16 and page_size & (page_size - 1) == 0)
+
+
+def wide_launch_shape(n_rows: int, n_heads: int, max_kv: int):
+    """(keys per split, splits) of a launch of ``attention_wide``: one wave per (row, 16 heads, split), splits as long as
+    still give the chip about 2,048 waves, and no shorter than 64 keys."""
+    groups = -(-n_heads // 16)
+    splits = max(1, min(2048 // max(n_rows * groups, 1), -(-max_kv // 64)))
+    chunk = max(64, -(-(-(-max_kv // splits)) // 32) * 32)
+    return chunk, max(1, -(-max_kv // chunk))
+
+
+def attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor, positions: torch.Tensor,
+                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int) -> torch.Tensor:
+    """Causal (optionally windowed) attention of q [T, nH, d] over one shared kv head with keys of d and values of dv
+    elements (K [pages, 1, page, d], V [pages, 1, dv, page]) on the matrix cores, for widths the other matrix-core kernels
+    do not take; returns [T, nH * dv].  Every row's keys are cut into splits of ``chunk`` (``max_splits`` * chunk must
+    reach past the largest position) and merged by a second launch."""
+    _check(q, "q", (None, None, None), torch.bfloat16)
+    T, nH, d = q.shape
+    _check(k_cache, "k_cache", (None, 1, None, d), torch.bfloat16)
+    n_pages, _, page_size, _ = k_cache.shape
+    _check(v_cache, "v_cache", (n_pages, 1, None, page_size), torch.bfloat16)
+    dv = v_cache.shape[2]
+    if not wide_attention_supported(q.dtype, 1, d, dv, page_size):
+        raise KernelError(f"attention_wide: keys of {d} (a multiple of 8 up to {WIDE_MAX_K_DIM}), values of {dv} (of 16 up to "
+                          f"{WIDE_MAX_V_DIM}), pages of {page_size} (a power of two from 16)")
+    _check(row_req, "row_req", (T,), torch.int32)
+    _check(positions, "positions", (T,), torch.int32)
+    _check(block_table, "block_table", (None, None), torch.int32)
+    out = torch.empty((T, nH * dv), dtype=torch.bfloat16, device=q.device)
+    part_o = torch.empty((T, nH, max_splits, dv), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((T, nH, max_splits, 2), dtype=torch.float32, device=q.device)
+    _call(load_module("attn_wide", (("K_DIM", d), ("V_DIM", dv))), "ifx_attn_wide",
+          (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P),
+          q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), 0, row_req.data_ptr(), positions.data_ptr(),
+          block_table.data_ptr(), block_table.shape[1], T, nH, d, dv, page_size, int(window or 0), int(chunk), int(max_splits),
+          float(scale), part_o.data_ptr(), part_ml.data_ptr(), _stream())
     return out
 
 

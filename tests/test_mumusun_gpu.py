@@ -297,6 +297,21 @@ def test_attention_over_a_latent_cache_at_the_windows_edges(dtype, n, window, d,
         assert (want[p, :dv] - v_in).abs().max() < 0.05 * v_in.abs().max()
 
 
+@pytest.mark.parametrize("n,window,d,dv,nH", [(70, 20, 40, 32, 3), (150, 33, 64, 48, 2), (200, 64, 48, 32, 4), (130, None, 56, 48, 20),
+                                              (100, 16, 64, 48, 16), (300, 72, 576, 512, 16), (530, 100, 136, 96, 33)])
+def test_wide_attention_on_the_matrix_cores(n, window, d, dv, nH):
+    """The same cases through the kernel for one shared kv head of any width, with the keys cut into splits of several
+    lengths (a split's edge inside a page, inside the window, past the end)."""
+    q, kc, vc, table, want = _paged_case("bfloat16", n, window, d, dv, nH)
+    row_req, pos = torch.zeros(n, dtype=torch.int32, device=DEV), torch.arange(n, dtype=torch.int32, device=DEV)
+    bound = table.shape[1] * 16
+    for chunk in (32, 96, 64 * -(-bound // 64)):
+        got = ops.attention_wide(q.to(DEV), kc.to(DEV), vc.to(DEV), row_req, pos, table.to(DEV), window, 1.0, chunk, -(-bound // chunk)).cpu()
+        assert rel_err(got, want) < 2e-2, chunk
+    chunk, splits = ops.wide_launch_shape(n, nH, bound)
+    assert chunk % 32 == 0 and chunk * splits >= bound
+
+
 # ---- the model through the step function ----------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(mm.CONFIGS))
