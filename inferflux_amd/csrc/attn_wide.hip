@@ -6,8 +6,9 @@
 // heads are the columns of the matrix tile, so a key or value is fetched once for all of them.  Their queries wait in
 // LDS (16 x K_DIM bf16, read as the second operand of the score product step by step), which leaves the registers to
 // the output: V_DIM / 16 tiles of four floats per lane.  Scores, softmax and the layout of both products are
-// attn_mfma.hip's row kernel's (S^T[key, head] = K Q^T; O^T[dim, head] += V^T P^T), as are the splits' partial results
-// and the launch that merges them (attn_shared.h, built here for the values' width).
+// attn_mfma.hip's row kernel's (S^T[key, head] = K Q^T; O^T[dim, head] += V^T P^T), as is the form of the splits' partial
+// results; a launch of its own merges them (a wave per (row, head), a lane a run of four elements), and a row in one
+// split writes its output itself.
 //
 // Compile with -DK_DIM=<multiple of 8> -DV_DIM=<multiple of 16>.
 #include "common.h"
@@ -72,12 +73,15 @@ __global__ __launch_bounds__(WAVE) void attn_wide_rows_kernel(RowArgs a) {
       vp[t] = a.v_cache + ((size_t)(lv ? page : 0) * D + col) * P + off + 4 * g4;
       s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
       if (lv) {
-#pragma unroll 6
+        // all of the tile's key pieces are asked for before the first product (a chain of trips to memory otherwise)
+        bf16x8 kop[KSK];
+#pragma unroll
+        for (int ks = 0; ks < KSK; ++ks) kop[ks] = 32 * ks + 8 * g4 < DK ? *(const bf16x8*)(kp + 32 * ks) : zero8();
+#pragma unroll
         for (int ks = 0; ks < KSK; ++ks) {
           const int c = 32 * ks + 8 * g4;
-          const bf16x8 kop = c < DK ? *(const bf16x8*)(kp + 32 * ks) : zero8();
           const bf16x8 qop = c < DK ? *(const bf16x8*)&qs[col * QP + c] : zero8();
-          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop, s[t], 0, 0, 0);
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[ks], qop, s[t], 0, 0, 0);
         }
       }
 #pragma unroll
@@ -104,20 +108,87 @@ __global__ __launch_bounds__(WAVE) void attn_wide_rows_kernel(RowArgs a) {
     l = l * alpha + psum;
     m = m_new;
     const bf16x8 pop = join4(pb[0], pb[1]);
-#pragma unroll 8
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16x4 v0 = live[0] ? *(const bf16x4*)(vp[0] + (size_t)16 * dt * P) : zero4();
-      const bf16x4 v1 = live[1] ? *(const bf16x4*)(vp[1] + (size_t)16 * dt * P) : zero4();
+    constexpr int VB = DT < 8 ? DT : 8;       // value tiles whose pieces are asked for together
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join4(v0, v1), pop, o[dt], 0, 0, 0);
+    for (int d0 = 0; d0 < DT; d0 += VB) {
+      bf16x4 v0[VB], v1[VB];
+#pragma unroll
+      for (int i = 0; i < VB; ++i) {
+        const int dt = d0 + i;
+        v0[i] = (live[0] && dt < DT) ? *(const bf16x4*)(vp[0] + (size_t)16 * dt * P) : zero4();
+        v1[i] = (live[1] && dt < DT) ? *(const bf16x4*)(vp[1] + (size_t)16 * dt * P) : zero4();
+      }
+#pragma unroll
+      for (int i = 0; i < VB; ++i) {
+        const int dt = d0 + i;
+        if (dt < DT) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join4(v0[i], v1[i]), pop, o[dt], 0, 0, 0);
+        }
+      }
     }
   }
   l = col_sum(l);
-  if (head_ok) {
-    if (g4 == 0) { pml[0] = m; pml[1] = l; }
+  if (!head_ok) return;
+  if (a.max_splits == 1) {      // the row's only split: the output itself, no partial result and no merge
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* orow = a.out + ((size_t)row * a.nH + head) * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = o[dt];
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x4 y;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) y[r] = (__bf16)(o[dt][r] * inv);
+      *(bf16x4*)(orow + 16 * dt + 4 * g4) = y;
+    }
+    return;
+  }
+  if (g4 == 0) { pml[0] = m; pml[1] = l; }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = o[dt];
+}
+
+// out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits in ascending order, M = max m_s.
+// One wave per (row, head); a lane owns runs of four output elements.
+__global__ __launch_bounds__(WAVE) void attn_wide_merge_kernel(RowArgs a) {
+  constexpr int C4 = (D + 255) / 256;
+  const int ri = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int row = a.rows ? a.rows[ri] : ri;
+  const float* po = a.part_o + ((size_t)ri * a.nH + head) * a.max_splits * D;
+  const float* pml = a.part_ml + ((size_t)ri * a.nH + head) * a.max_splits * 2;
+  float M = -INFINITY;
+  for (int s = lane; s < a.max_splits; s += WAVE) M = fmaxf(M, pml[2 * s]);
+  M = wave_max(M);
+  floatx4 acc[C4];
+#pragma unroll
+  for (int c = 0; c < C4; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float L = 0.f;
+  for (int s = 0; s < a.max_splits; ++s) {
+    const float ms = pml[2 * s];
+    if (ms == -INFINITY) continue;          // uniform over the wave: a split without a visible key
+    const float w = fast_exp2(ms - M);
+    L += w * pml[2 * s + 1];
+#pragma unroll
+    for (int c = 0; c < C4; ++c) {
+      const int e = 4 * lane + 256 * c;
+      if (e < D) {
+        const floatx4 v = *(const floatx4*)(po + (size_t)s * D + e);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[c][r] += w * v[r];
+      }
+    }
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  bf16_t* orow = a.out + ((size_t)row * a.nH + head) * D;
+#pragma unroll
+  for (int c = 0; c < C4; ++c) {
+    const int e = 4 * lane + 256 * c;
+    if (e < D) {
+      bf16x4 y;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) y[r] = (__bf16)(acc[c][r] * inv);
+      *(bf16x4*)(orow + e) = y;
+    }
   }
 }
 
@@ -139,6 +210,6 @@ extern "C" int ifx_attn_wide(const void* q, const void* k_cache, const void* v_c
             scale * 1.4426950408889634f, 0, 0, 0};
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_wide_rows_kernel, dim3(max_splits, (nH + 15) / 16, n_rows), dim3(WAVE), (size_t)16 * QP * sizeof(bf16_t), s, a);
-  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, a);
+  if (max_splits > 1) hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);
   IFX_LAUNCH_CHECK();
 }
