@@ -87,7 +87,7 @@ def write_model(folder, cfg, seed, gain=4.0, decisive_router=False):
                 t = t * spec.shape[-1] ** 0.5
         tensors[name] = t.to(torch.bfloat16).contiguous()
     if decisive_router:
-        n = max(L["mlp"]["router"]["experts"] for L in cfg["layers"] if L["mlp"] is not None)
+        n = max([L["mlp"]["router"]["experts"] for L in cfg["layers"] if L["mlp"] is not None], default=0)
         values = torch.tensor(router_values(n))
         for tok in range(cfg["vocab"]):
             tensors["embed"][tok, :n] = values[torch.randperm(n, generator=g)].to(torch.bfloat16)

@@ -455,6 +455,49 @@ def test_replay_of_traces_with_pages_and_slots_used_again(name, dtype, folders, 
         assert rel_err(got, want) < TOL[dtype], (step, rows[:3])
 
 
+def _drawn_config(seed):
+    """A configuration drawn from sizes of every kind: latents that the matrix-core attention kernels take whole (a multiple of
+    16 up to 128), that the kernel for one shared kv head takes, and that only the plain kernel takes; more heads than a matrix
+    tile has columns; layers with and without window and feed-forward; routers with and without groups."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([48, 72, 96, 160])
+    layers = []
+    for _ in range(rng.choice([1, 2, 3])):
+        kv_rank, rot_dim = rng.choice([(16, 16), (48, 16), (64, 16), (96, 32), (96, 16), (32, 8), (80, 24), (20, 6), (136, 8)])
+        dims = rng.choice([rot_dim, max(2, rot_dim // 2 // 2 * 2)])
+        mixer = mm._mixer(rng.choice([1, 2, 5, 8, 20]), rng.choice([8, 12, 16, 40]), rot_dim, rng.choice([8, 10, 24, 48]), rng.choice([16, 24, 52]),
+                          kv_rank, rng.choice([0.1, 0.17, 0.3]), rng.choice([100.0, 10000.0, 1e6]), dims, rng.choice([None, 5, 16, 17, 64, 100]))
+        count = rng.choice([1, 2, 3, 4])
+        per = rng.choice([1, 2, 3])
+        keep = rng.randint(1, count)
+        mlp = rng.choice([None, mm._moe(count * per, rng.randint(1, keep * per), rng.choice([16, 24, 48, 80]), count, keep)])
+        layers.append(mm._layer(mixer, mlp))
+    return {"architecture": "Mumusun", "vocab": rng.choice([61, 128, 500]), "width": width, "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])},
+            "layers": layers}
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations(seed, tmp_path):
+    """Whole prompts, portions and decoding of drawn configurations against the plain implementation, both precisions."""
+    cfg = _drawn_config(seed)
+    for dtype in ("float32", "bfloat16"):
+        folder = mm.write_model(str(tmp_path / dtype), cfg, 80 + seed, gain=GAIN[dtype], decisive_router=dtype == "bfloat16")
+        runner = load_runner(folder, DT[dtype], num_pages=24, max_requests=3)
+        ids = ids_of(seed, 150, cfg["vocab"])
+        want = plain(folder, ids)
+        assert rel_err(run_whole(runner, "w", ids), want) < TOL[dtype], (seed, dtype, cfg)
+        runner.add_request("c")
+        runner.add_request("other")
+        rows, p = [], 0
+        for m in [33, 2, 64, 1, 1, 17, 1, 1, 1, 29]:
+            out = runner.step([StepEntry("other", ids_of(p, 3, cfg["vocab"]), []), StepEntry("c", ids[p:p + m], list(range(m)))]).cpu()
+            rows.append(out)
+            p += m
+        assert p == len(ids) and rel_err(torch.cat(rows), want) < TOL[dtype], (seed, dtype, cfg)
+        runner.manager.check()
+
+
 # ---- generation through the engine's own entry point and scheduler ------------------------------
 @pytest.mark.parametrize("name", ["P", "R"])
 def test_greedy_generation_through_the_engine(name, folders):
