@@ -29,7 +29,7 @@ CONFIGS = {
     "P": {"architecture": "Mumusun", "vocab": 300, "width": 64, "norm": {"eps": 1e-5}, "layers": [
         _layer(_mixer(3, 16, 8, 24, 40, 32, 0.2, 10000.0, window=20), _moe(8, 3, 48, 4, 2)),
         _layer(_mixer(2, 8, 16, 8, 16, 48, 0.25, 500.0, dims=8, window=33), None),
-        _layer(_mixer(4, 24, 4, 12, 24, 40, 0.19, 250000.0), _moe(6, 1, 40)),
+        _layer(_mixer(4, 24, 4, 12, 24, 40, 0.19, 300000.0), _moe(6, 1, 40)),
     ]},
     # one head, one group kept of three, top 2, widths that are no multiples of 8 or 16, a window shorter than a page
     "Q": {"architecture": "Mumusun", "vocab": 131, "width": 88, "norm": {"eps": 1e-6}, "layers": [

@@ -165,7 +165,7 @@ def test_headwise_product_with_rotated_tail(dtype, T, H, K, N, tail, rot):
     assert rel_err(got, want) < (1e-5 if dtype == "float32" else 1e-2)
 
 
-@pytest.mark.parametrize("E,top,count,keep", [(8, 3, 4, 2), (12, 4, 2, 1), (6, 1, 1, 1), (9, 2, 3, 1), (4, 4, 2, 2), (16, 2, 16, 5), (64, 6, 8, 3)])
+@pytest.mark.parametrize("E,top,count,keep", [(8, 3, 4, 2), (10, 3, 2, 1), (6, 1, 1, 1), (9, 2, 3, 1), (4, 4, 2, 2), (16, 2, 16, 5), (64, 6, 8, 3)])
 def test_router_scores_groups_and_choice(E, top, count, keep):
     T, K = 50, 72
     h, w = rnd(10, T, K), rnd(11, E, K, scale=0.4)
@@ -284,7 +284,7 @@ def _paged_case(dtype, n, window, d, dv, nH, P=16, seed=20):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n,window,d,dv,nH", [(70, 20, 40, 32, 3), (150, 33, 64, 48, 2), (40, 7, 56, 44, 1), (200, 64, 48, 32, 4),
-                                              (130, None, 44, 40, 4), (100, 16, 64, 48, 16), (530, 72, 128, 96, 6)])
+                                              (130, None, 44, 40, 4), (100, 16, 64, 48, 16), (530, 90, 120, 88, 5)])
 def test_attention_over_a_latent_cache_at_the_windows_edges(dtype, n, window, d, dv, nH):
     """Keys as wide as latent + rotated part, values as wide as the latent, one shared kv head."""
     q, kc, vc, table, want = _paged_case(dtype, n, window, d, dv, nH)
@@ -298,7 +298,7 @@ def test_attention_over_a_latent_cache_at_the_windows_edges(dtype, n, window, d,
 
 
 @pytest.mark.parametrize("n,window,d,dv,nH", [(70, 20, 40, 32, 3), (150, 33, 64, 48, 2), (200, 64, 48, 32, 4), (130, None, 56, 48, 20),
-                                              (100, 16, 64, 48, 16), (300, 72, 576, 512, 16), (530, 100, 136, 96, 33)])
+                                              (100, 16, 64, 48, 16), (300, 80, 576, 512, 16), (530, 100, 136, 96, 33)])
 def test_wide_attention_on_the_matrix_cores(n, window, d, dv, nH):
     """The same cases through the kernel for one shared kv head of any width, with the keys cut into splits of several
     lengths (a split's edge inside a page, inside the window, past the end)."""
