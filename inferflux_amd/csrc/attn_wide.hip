@@ -29,7 +29,7 @@ constexpr int QP = DK + 8;              // elements per query row in LDS (the pa
 
 extern "C" int ifx_attn_wide_dims() { return DK * 1024 + D; }
 
-__global__ __launch_bounds__(WAVE) void attn_wide_rows_kernel(RowArgs a) {
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_wide_rows_kernel(RowArgs a) {
   extern __shared__ __attribute__((aligned(16))) bf16_t qs[];      // [16][QP]
   const int split = blockIdx.x, hg = blockIdx.y, ri = blockIdx.z;
   const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
@@ -91,6 +91,8 @@ __global__ __launch_bounds__(WAVE) void attn_wide_rows_kernel(RowArgs a) {
         s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
         mb = fmaxf(mb, s[t][r]);
       }
+      // one tile's key pieces at a time: both tiles' together cost 72 registers more and the second wave of a SIMD its place
+      __builtin_amdgcn_sched_barrier(0);
     }
     const float m_new = fmaxf(m, col_max(mb));
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
