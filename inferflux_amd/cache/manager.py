@@ -10,7 +10,8 @@ Layers whose mixers keep the same kind of history form a *group*: all layers tha
 key share one group, all layers that keep a window of W keys share another.  Each group has
 its own pool of pages and, for every request, its own block table: entry b is the page that
 holds positions [b * page_size, (b + 1) * page_size) for every layer of the group, or -1 once
-a windowed group has given that page back.
+a windowed group has given that page back.  A windowed group may also keep a request's first
+positions for good (``keep_first``: queries that see a window and the first tokens beside it).
 
 A request's life: ``add`` (takes a state slot), then per step ``reserve(n)`` (pages for its
 next n positions in every group, all or nothing) and, after the step ran, ``commit(n)``
@@ -53,9 +54,11 @@ class OutOfSlots(RuntimeError):
 
 @dataclasses.dataclass(frozen=True)
 class GroupSpec:
-    """A set of schedule entries whose caches share pages.  ``window`` None keeps everything."""
+    """A set of schedule entries whose caches share pages.  ``window`` None keeps everything; a windowed group
+    still keeps the pages that hold any of the first ``keep_first`` positions of a request."""
     window: Optional[int]
     entries: Tuple[int, ...]
+    keep_first: int = 0
 
 
 @dataclasses.dataclass
@@ -79,7 +82,7 @@ class _Native:
             mod = load_module("cache_manager")
             ip = ctypes.POINTER(ctypes.c_int)
             sig = {
-                "cm_create": ((I, ip, ip, I, I), P), "cm_destroy": ((P,), None),
+                "cm_create": ((I, ip, ip, I, I), P), "cm_destroy": ((P,), None), "cm_set_keep_first": ((P, I, I), I),
                 "cm_pool_num_pages": ((P, I), I), "cm_pool_num_free": ((P, I), I), "cm_pool_take": ((P, I), I),
                 "cm_pool_retain": ((P, I, I), I), "cm_pool_release": ((P, I, I), I), "cm_pool_refs": ((P, I, I), I),
                 "cm_pool_free_list": ((P, I, ip), I), "cm_free_slots": ((P,), I), "cm_add": ((P,), I),
@@ -175,6 +178,9 @@ class CacheManager:
         self._h = self._n.cm_create(len(counts), _ints(counts), _ints(windows), page_size, max_requests)
         if not self._h:
             raise ValueError(self._n.last_error())
+        for g, spec in enumerate(self.groups):
+            if spec.keep_first and spec.window is not None and self._n.cm_set_keep_first(self._h, g, int(spec.keep_first)) != 0:
+                raise ValueError(self._n.last_error())
         self.pools = [PagePool(n, _owner=self._h, _group=g) for g, n in enumerate(counts)]
         self.max_requests = max_requests
         self._slot: Dict[Hashable, int] = {}        # live request -> its slot, which is how the native side knows it

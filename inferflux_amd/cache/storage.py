@@ -27,14 +27,15 @@ def plan_groups(schedule, mixers) -> Tuple[List[GroupSpec], Dict[int, int]]:
     ``mixers[i]`` is the mixer schedule entry i runs.  Returns the groups and, for every entry
     that touches a cache (its own or another's), the group it belongs to.
     """
-    by_window: Dict[Optional[int], List[int]] = {}
+    by_window: Dict[Tuple[Optional[int], int], List[int]] = {}
     for i, e in enumerate(schedule):
         spec = mixers[i].cache_spec()
         if spec is None or e.cache_from is not None:
             continue
-        by_window.setdefault(spec.window, []).append(i)
-    keys = sorted(by_window, key=lambda w: (w is not None, w or 0))
-    groups = [GroupSpec(window=w, entries=tuple(by_window[w])) for w in keys]
+        # (what a mixer that keeps everything calls its first positions changes nothing about its pages)
+        by_window.setdefault((spec.window, spec.keep_first if spec.window is not None else 0), []).append(i)
+    keys = sorted(by_window, key=lambda wk: (wk[0] is not None, wk[0] or 0, wk[1]))
+    groups = [GroupSpec(window=w, entries=tuple(by_window[(w, k)]), keep_first=k) for w, k in keys]
     entry_group = {i: g for g, spec in enumerate(groups) for i in spec.entries}
     for i, e in enumerate(schedule):
         if e.cache_from is not None and mixers[i].cache_spec() is not None:
@@ -42,8 +43,9 @@ def plan_groups(schedule, mixers) -> Tuple[List[GroupSpec], Dict[int, int]]:
             mine = mixers[i].cache_spec()
             if owner is None or (owner.n_kv_heads, owner.k_dim, owner.v_dim) != (mine.n_kv_heads, mine.k_dim, mine.v_dim):
                 raise ValueError(f"schedule[{i}] reads the cache of entry {e.cache_from}, whose shape differs")
-            if owner.window is not None and (mine.window is None or mine.window > owner.window):
-                raise ValueError(f"schedule[{i}] reads further back than entry {e.cache_from} keeps (window {owner.window})")
+            if owner.window is not None and (mine.window is None or mine.window > owner.window or mine.keep_first > owner.keep_first):
+                raise ValueError(f"schedule[{i}] reads further back than entry {e.cache_from} keeps (window {owner.window}, "
+                                 f"first {owner.keep_first})")
             entry_group[i] = entry_group[e.cache_from]
     return groups, entry_group
 

@@ -11,6 +11,11 @@
 // the query at position p sees keys j with max(0, p - window + 1) <= j <= p; s_j = (q . k_j) *
 // scale; o = sum_j softmax(s)_j v_j.
 //
+// Three further parameters, each off when zero: ``keep_first``, the first positions of a request that a windowed
+// query still sees beside its window (j <= p and (p - j < window or j < keep_first)), at their true positions;
+// ``has_sink``, a key without value whose score is ``sink_score`` and which only takes part in the softmax's
+// denominator (with score 0: p_j = exp(s_j) / (1 + sum exp(s_j))); ``gate`` [T, nH], a factor on each head's output.
+//
 // Cache layouts: K [page][kv head][offset][d], V [page][kv head][dv][offset].  Values may have another width
 // than keys (dv != d): the output row of a head then has dv elements.
 #include "common.h"
@@ -44,6 +49,10 @@ struct AttnArgs {
   int max_blocks;
   int T, nH, nKV, d, dv, page_size, window;
   float scale;
+  int keep_first;
+  int has_sink;
+  float sink_score;
+  const float* gate;
 };
 
 template <typename T>
@@ -60,6 +69,7 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
   const int pos = a.positions[row];
   const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int keep = lo > 0 ? min(a.keep_first, lo) : 0;      // keys [0, keep) and [lo, pos] are seen
 
   const T* qrow = (const T*)a.q + ((size_t)row * a.nH + head) * d;
   for (int e = lane; e < d; e += WAVE) q_s[wid][e] = to_f(qrow[e]);
@@ -67,16 +77,21 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_s_waitcnt(0);
 
-  float m = -INFINITY, l = 0.f;
+  // (the sink is a key of score sink_score whose value is zero: it starts the running maximum and sum)
+  float m = a.has_sink ? a.sink_score : -INFINITY, l = a.has_sink ? 1.f : 0.f;
   float acc[DC];
 #pragma unroll
   for (int c = 0; c < DC; ++c) acc[c] = 0.f;
 
   const T* Kc = (const T*)a.k_cache;
   const T* Vc = (const T*)a.v_cache;
-  for (int t0 = (lo / WAVE) * WAVE; t0 <= pos; t0 += WAVE) {
+  for (int t0 = keep > 0 ? 0 : (lo / WAVE) * WAVE; t0 <= pos; t0 += WAVE) {
+    if (t0 >= keep && t0 + WAVE <= lo) {     // between the kept first keys and the window: on to the window's first tile
+      t0 = (lo / WAVE) * WAVE - WAVE;
+      continue;
+    }
     const int j = t0 + lane;
-    const bool valid = j >= lo && j <= pos;
+    const bool valid = (j >= lo || j < keep) && j <= pos;
     int page = 0, off = 0;
     float s = -INFINITY;
     if (valid) {
@@ -96,7 +111,7 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
       }
       s = dot * a.scale;
     }
-    const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds key `lo` or later, up to pos
+    const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds a visible key
     const float p = valid ? expf(s - m_new) : 0.f;
     const float alpha = expf(m - m_new);  // 0 on the first tile (m = -inf)
     l = l * alpha + wave_sum(p);
@@ -108,7 +123,7 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
       // not finite) add nothing; an element's sum still runs over the keys in ascending order.
       for (int g = 0; g < WAVE; g += 8) {
         const int j0 = t0 + g;
-        if (j0 > pos || j0 + 7 < lo) continue;                  // uniform over the wave
+        if (j0 > pos || (j0 + 7 < lo && j0 >= keep)) continue;  // uniform over the wave
         float pj[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) pj[i] = __shfl(p, g + i, WAVE);
@@ -139,7 +154,7 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
     m = m_new;
   }
   T* orow = (T*)a.out + ((size_t)row * a.nH + head) * dv;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float inv = (l > 0.f ? 1.f / l : 0.f) * (a.gate ? a.gate[(size_t)row * a.nH + head] : 1.f);
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
     const int e = lane + c * WAVE;
@@ -150,13 +165,14 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
 extern "C" int ifx_attn_plain(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                               const int* row_req, const int* positions, const int* block_table,
                               int max_blocks, int T, int nH, int nKV, int d, int dv, int page_size, int window,
-                              float scale, void* stream) {
+                              float scale, int keep_first, int has_sink, float sink_score, const float* gate, void* stream) {
+  IFX_REQUIRE(keep_first >= 0, "attn_plain: keep_first %d", keep_first);
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_plain: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(d > 0 && d <= MAX_D, "attn_plain: head_dim %d outside 1..%d", d, MAX_D);
   IFX_REQUIRE(dv > 0 && dv <= MAX_D, "attn_plain: value head_dim %d outside 1..%d", dv, MAX_D);
   IFX_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attn_plain: bad page_size/max_blocks/window");
   if (T == 0) return 0;
-  AttnArgs a{q, k_cache, v_cache, out, row_req, positions, block_table, max_blocks, T, nH, nKV, d, dv, page_size, window, scale};
+  AttnArgs a{q, k_cache, v_cache, out, row_req, positions, block_table, max_blocks, T, nH, nKV, d, dv, page_size, window, scale, keep_first, has_sink, sink_score, gate};
   const long long items = (long long)T * nH;
   const unsigned blocks = (unsigned)((items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
   hipStream_t s = (hipStream_t)stream;

@@ -4,7 +4,8 @@
 // A request is known here by its state slot (0 .. max_requests - 1), which it holds from add to free.
 // Groups: entry g of ``windows`` is the number of positions the group's layers look back (-1: all of them);
 // a windowed group gives a page back as soon as every position in it lies before the window of the next
-// query.  Pages are handed out most recently freed first; a page returns to its pool when its reference
+// query, except the pages that hold any of the group's first ``keep_first`` positions (set per group with
+// cm_set_keep_first; 0 unless set), which every later query still reads.  Pages are handed out most recently freed first; a page returns to its pool when its reference
 // count reaches zero.  Every call either succeeds or changes nothing.
 //
 // The reference accounts pages on the host in the same units (16-token blocks with reference counts:
@@ -53,6 +54,7 @@ struct Manager {
   int page_size, max_requests;
   std::vector<Pool> pools;
   std::vector<int> windows;
+  std::vector<int> keep_first;   // per group: positions from the start that a windowed group never gives back
   std::vector<int> free_slots;   // back() is handed out next
   std::vector<Request> requests;
   long long epochs = 0;
@@ -92,6 +94,7 @@ void* cm_create(int n_groups, const int* num_pages, const int* windows, int page
   for (int g = 0; g < n_groups; ++g) {
     m->pools.emplace_back(num_pages[g]);
     m->windows.push_back(windows[g]);
+    m->keep_first.push_back(0);
   }
   for (int s = max_requests - 1; s >= 0; --s) m->free_slots.push_back(s);   // slot 0 first
   m->requests.resize(max_requests);
@@ -99,6 +102,15 @@ void* cm_create(int n_groups, const int* num_pages, const int* windows, int page
 }
 
 void cm_destroy(void* h) { delete (Manager*)h; }
+
+// The first ``n`` positions of every request stay readable in group g whatever its window (before any request is added).
+int cm_set_keep_first(void* h, int g, int n) {
+  Manager* m = (Manager*)h;
+  if (g < 0 || g >= (int)m->pools.size() || n < 0) FAIL(-1, "keep_first %d for group %d of %d", n, g, (int)m->pools.size());
+  if ((int)m->free_slots.size() != m->max_requests) FAIL(-1, "keep_first is set before any request is added");
+  m->keep_first[g] = n;
+  return 0;
+}
 
 // ---- pools ----------------------------------------------------------------------------------------------
 int cm_pool_num_pages(void* h, int g) { return ((Manager*)h)->pools[g].num_pages; }
@@ -232,7 +244,8 @@ int cm_commit(void* h, int slot, int n_new) {
     if (first_needed <= 0) continue;
     std::vector<int>& t = r->tables[g];
     const int dead = std::min(first_needed / m->page_size, (int)t.size());
-    for (int b = dead - 1; b >= 0; --b) {   // released blocks form a prefix: stop at the first -1
+    const int kept = m->blocks_for(m->keep_first[g]);   // blocks that hold a kept first position are never given back
+    for (int b = dead - 1; b >= kept; --b) {   // released blocks form a run behind the kept ones: stop at the first -1
       if (t[b] < 0) break;
       m->pools[g].release(t[b]);
       t[b] = -1;

@@ -15,32 +15,32 @@
 IFX_DEFINE_LAST_ERROR()
 
 // ---------------------------------------------------------------------------------------
-// out[t, :] = float(table[ids[t], :])
+// out[t, :] = float(table[ids[t], :]) * scale
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                 float* __restrict__ out, int H) {
+                                 float* __restrict__ out, int H, float scale) {
   // (a row is cut into runs of 4,096 columns, one workgroup each: rows as wide as a vocabulary then fill the chip too)
   const int t = blockIdx.x, i0 = blockIdx.y * 4096, i1 = min(H, i0 + 4096);
   const T* src = table + (size_t)ids[t] * H;
   float* dst = out + (size_t)t * H;
-  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) dst[i] = to_f(src[i]);
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) dst[i] = to_f(src[i]) * scale;
 }
 
 extern "C" int ifx_embedding(const int* ids, const void* table, int table_dtype, float* out, int T,
-                             int H, void* stream) {
+                             int H, float scale, void* stream) {
   IFX_REQUIRE(T >= 0 && H > 0, "embedding: bad sizes T=%d H=%d", T, H);
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (table_dtype == DT_F32)
-    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const float*)table, out, H);
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const float*)table, out, H, scale);
   else if (table_dtype == DT_BF16)
-    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const bf16_t*)table, out, H);
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const bf16_t*)table, out, H, scale);
   else
     IFX_FAIL("embedding: unknown dtype %d", table_dtype);
   IFX_LAUNCH_CHECK();
 }
 
-// The same for up to 16 tokens, with what the RMS norm that reads the stream first needs written beside it, so that
+// The same (times ``scale``) for up to 16 tokens, with what the RMS norm that reads the stream first needs written beside it, so that
 // the norm takes no kernel of its own: rows[t, :] = bf16(out[t, :] * norm_w[:]) and pieces[run][t] = the sum of the
 // squares of out[t, :] over run ``run`` of 4,096 columns (zero for t >= n_rows; ``pieces`` is [runs][16]).  The
 // product that reads ``rows`` multiplies its sums by rsqrt(sum of the pieces / H + eps) (RowScale in gemm_bf16.hip).
@@ -48,14 +48,14 @@ template <typename T>
 __global__ __launch_bounds__(256) void embedding_norm_kernel(const int* __restrict__ ids, const T* __restrict__ table,
                                                             const bf16_t* __restrict__ norm_w, float* __restrict__ out,
                                                             bf16_t* __restrict__ rows, float* __restrict__ pieces,
-                                                            int n_rows, int H) {
+                                                            int n_rows, int H, float scale) {
   __shared__ float red[16];
   const int t = blockIdx.x, run = blockIdx.y, i0 = run * 4096, i1 = min(H, i0 + 4096);
   float ss = 0.f;
   if (t < n_rows) {
     const T* src = table + (size_t)ids[t] * H;
     for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) {
-      const float x = to_f(src[i]);
+      const float x = to_f(src[i]) * scale;
       out[(size_t)t * H + i] = x;
       rows[(size_t)t * H + i] = (bf16_t)(x * to_f(norm_w[i]));
       ss += x * x;
@@ -66,29 +66,29 @@ __global__ __launch_bounds__(256) void embedding_norm_kernel(const int* __restri
 }
 
 extern "C" int ifx_embedding_norm(const int* ids, const void* table, int table_dtype, const void* norm_w, float* out,
-                                  void* rows, float* pieces, int T, int H, void* stream) {
+                                  void* rows, float* pieces, int T, int H, float scale, void* stream) {
   IFX_REQUIRE(T >= 0 && T <= 16 && H > 0, "embedding_norm: T=%d must be at most 16 (H=%d)", T, H);
   IFX_REQUIRE(norm_w && out && rows && pieces, "embedding_norm: needs the norm's weight and three outputs");
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(16, (H + 4095) / 4096);
   if (table_dtype == DT_F32)
-    hipLaunchKernelGGL(embedding_norm_kernel<float>, grid, dim3(256), 0, s, ids, (const float*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H);
+    hipLaunchKernelGGL(embedding_norm_kernel<float>, grid, dim3(256), 0, s, ids, (const float*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H, scale);
   else if (table_dtype == DT_BF16)
-    hipLaunchKernelGGL(embedding_norm_kernel<bf16_t>, grid, dim3(256), 0, s, ids, (const bf16_t*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H);
+    hipLaunchKernelGGL(embedding_norm_kernel<bf16_t>, grid, dim3(256), 0, s, ids, (const bf16_t*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H, scale);
   else
     IFX_FAIL("embedding_norm: unknown dtype %d", table_dtype);
   IFX_LAUNCH_CHECK();
 }
 
 // ---------------------------------------------------------------------------------------
-// x = residual[src] (+ delta[src]);  if write_back: residual[src] = x
+// x = residual[src] (+ delta_scale * delta[src]);  if write_back: residual[src] = x
 // out[r, :] = x * rsqrt(mean(x^2) + eps) * weight         src = rows ? rows[r] : r
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                    const void* __restrict__ weight, int weight_dtype,
                                    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps,
-                                   int write_back, int n_slices, size_t slice_stride) {
+                                   int write_back, int n_slices, size_t slice_stride, float delta_scale) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -98,7 +98,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   auto delta_at = [&](int i) {
     float d = to_f(dl[i]);
     for (int s = 1; s < n_slices; ++s) d += to_f(dl[(size_t)s * slice_stride + i]);
-    return d;
+    return d * delta_scale;
   };
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
@@ -148,7 +148,8 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const floa
 template <typename TD, typename TO, typename TW, int NV>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                               const TW* __restrict__ weight, TO* __restrict__ out,
-                                                              const int* __restrict__ rows, int H, float eps, int write_back) {
+                                                              const int* __restrict__ rows, int H, float eps, int write_back,
+                                                              float delta_scale) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         float d4[4];
         load4<TD>(dl + i, d4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) x[v][e] += d4[e];
+        for (int e = 0; e < 4; ++e) x[v][e] += d4[e] * delta_scale;
         if (write_back) store4<float>(res + i, x[v]);
       }
 #pragma unroll
@@ -195,7 +196,7 @@ template <typename TD, typename TO, typename TW, int NV>
 __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                               const TW* __restrict__ weight, TO* __restrict__ out,
                                                               const int* __restrict__ rows, int H, float eps, int write_back,
-                                                              int n_slices, size_t slice_stride) {
+                                                              int n_slices, size_t slice_stride, float delta_scale) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restri
     for (int v = 0; v < NV; ++v) {
       const int i = 4 * (threadIdx.x + 256 * v);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[v][e] += d4[v][e];
+      for (int e = 0; e < 4; ++e) x[v][e] += d4[v][e] * delta_scale;
       if (write_back && i < H) store4<float>(res + i, x[v]);
     }
   }
@@ -268,15 +269,16 @@ __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restri
 
 template <typename TD, typename TO, typename TW>
 static void launch_rmsnorm_vec(float* residual, const void* delta, const void* weight, void* out, const int* rows,
-                               int n_rows, int H, float eps, int write_back, int n_slices, size_t slice_stride, hipStream_t s) {
+                               int n_rows, int H, float eps, int write_back, int n_slices, size_t slice_stride, float delta_scale,
+                               hipStream_t s) {
 #define GO(NV_)                                                                                                              \
   do {                                                                                                                       \
     if (n_slices > 1)                                                                                                        \
       hipLaunchKernelGGL((add_rmsnorm_slices_kernel<TD, TO, TW, NV_>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta, \
-                         (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);                      \
+                         (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride, delta_scale);         \
     else                                                                                                                     \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, NV_>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta, \
-                         (const TW*)weight, (TO*)out, rows, H, eps, write_back);                                              \
+                         (const TW*)weight, (TO*)out, rows, H, eps, write_back, delta_scale);                                 \
   } while (0)
   if (H <= 4 * 256 * 2) GO(2);
   else if (H <= 4 * 256 * 4) GO(4);
@@ -285,9 +287,11 @@ static void launch_rmsnorm_vec(float* residual, const void* delta, const void* w
 }
 
 // n_slices > 1: ``delta`` (float32) holds that many partial sums, slice_stride elements apart, added in order.
+// ``delta_scale``: the factor on the delta (1 for the plain add; a model's factor on every sub-block's output).
 extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
                                int weight_dtype, void* out, int out_dtype, const int* rows, int n_rows,
-                               int H, float eps, int write_back, int n_slices, long long slice_stride, void* stream) {
+                               int H, float eps, int write_back, int n_slices, long long slice_stride, float delta_scale,
+                               void* stream) {
   IFX_REQUIRE(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
   IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || (delta && delta_dtype == DT_F32 && slice_stride > 0)),
               "add_rmsnorm: %d slices need a float32 delta and their distance", n_slices);
@@ -301,8 +305,8 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
   if (H % 4 == 0 && H <= 4 * 256 * 8) {
 #define VEC(TD, TO)                                                                                                  \
   do {                                                                                                               \
-    if (weight_dtype == DT_F32) launch_rmsnorm_vec<TD, TO, float>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, s); \
-    else launch_rmsnorm_vec<TD, TO, bf16_t>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, s);      \
+    if (weight_dtype == DT_F32) launch_rmsnorm_vec<TD, TO, float>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, delta_scale, s); \
+    else launch_rmsnorm_vec<TD, TO, bf16_t>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, delta_scale, s);      \
   } while (0)
     if (dd == DT_F32 && out_dtype == DT_F32) VEC(float, float);
     else if (dd == DT_BF16 && out_dtype == DT_BF16) VEC(bf16_t, bf16_t);
@@ -314,7 +318,7 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
   const int threads = H >= 2048 ? 512 : 256;
 #define LAUNCH(TD, TO)                                                                              \
   hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(threads), 0, s, residual,     \
-                     (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back, n_slices, (size_t)slice_stride)
+                     (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back, n_slices, (size_t)slice_stride, delta_scale)
   if (dd == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
   else if (dd == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
   else if (dd == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
@@ -324,23 +328,26 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
 }
 
 // ---------------------------------------------------------------------------------------
-// cos[t, p], sin[t, p] of angle = float(positions[t]) * inv_freq[p]: the step's rotation table, made
+// magnitude * cos[t, p], sin[t, p] of angle = float(positions[t]) * inv_freq[p]: the step's rotation table, made
 // once per step and read by every layer.
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                  float* __restrict__ cs, float* __restrict__ sn, int n_pairs, int n) {
+                                  float* __restrict__ cs, float* __restrict__ sn, int n_pairs, int n, float magnitude) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const int t = i / n_pairs, p = i % n_pairs;
-  sincosf((float)positions[t] * inv_freq[p], &sn[i], &cs[i]);
+  float sv, cv;
+  sincosf((float)positions[t] * inv_freq[p], &sv, &cv);
+  sn[i] = sv * magnitude;      // (a rotation with scaled frequencies may also lengthen what it turns: 1 otherwise)
+  cs[i] = cv * magnitude;
 }
 
 extern "C" int ifx_rope_table(const int* positions, const float* inv_freq, float* cs, float* sn, int T, int n_pairs,
-                              void* stream) {
+                              float magnitude, void* stream) {
   IFX_REQUIRE(T >= 0 && n_pairs > 0, "rope_table: bad sizes T=%d pairs=%d", T, n_pairs);
   if (T == 0) return 0;
   const int n = T * n_pairs;
   hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, positions, inv_freq, cs, sn,
-                     n_pairs, n);
+                     n_pairs, n, magnitude);
   IFX_LAUNCH_CHECK();
 }
 
@@ -350,6 +357,8 @@ extern "C" int ifx_rope_table(const int* positions, const float* inv_freq, float
 // (slot = page * page_size + offset; slot < 0: nothing is written to the cache).
 // Cache layouts: K [page][kv head][offset][d], V [page][kv head][dv][offset]; values may be
 // narrower or wider than keys (dv != d).
+// Optionally (see RopeArgs): q and k heads brought to unit root mean square after the rotation, the values mixed
+// with those of an earlier layer before they are cached, the projected values handed on, a sigmoid gate per head.
 // rope_style: 0 none, 1 split-half pairs (p, p + rot/2), 2 consecutive pairs (2p, 2p+1);
 // cos/sin come from the step's table [T, rotary_dim / 2]; elements at or beyond rotary_dim are
 // copied.  One block per (token, head): q heads, then k heads, then v heads.
@@ -369,13 +378,21 @@ struct RopeArgs {
   void* k_cache;
   void* v_cache;
   int dv;                // width of a value head
+  // What follows is optional (zero: absent).
+  int gate_cols;         // nH further columns behind q, k and v: sigmoid(x + bias) of column h goes to gate_out[t, h]
+  float* gate_out;       // [T, nH] float
+  int unit_norm;         // q and k heads are divided by their root mean square (+ norm_eps inside the root) after the rotation
+  float norm_eps;
+  const void* v_first;   // [T, nKV * dv] of the activation type: v <- (1 - v_mix) v + v_mix v_first before the cache write
+  float v_mix;
+  void* v_out;           // [T, nKV * dv]: the values as projected (with bias, before any mixing), for later layers to mix in
 };
 
 template <typename T>
 __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int t = blockIdx.x, head = blockIdx.y;
   const int d = a.d, dv = a.dv, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
-  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + kv_width + a.nKV * dv;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + kv_width + a.nKV * dv + a.gate_cols;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
   const float* part = (const float*)a.qkv + (size_t)t * row_width;
   // Elements i0 and i1 of the row; partial sums are added in slice order, eight slices of both elements asked for
@@ -400,11 +417,18 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int col = head * d;  // q heads, k heads and v heads follow each other in the row
   if (head < a.nH + a.nKV) {
     const bool is_q = head < a.nH;
+    if (is_q && a.gate_cols && threadIdx.x == 0) {      // the head's output gate, from the column behind q, k and v
+      const int gc = q_width + kv_width + a.nKV * dv + head;
+      float g, unused;
+      in2(gc, gc, g, unused);
+      if (a.bias) g += load_dyn(a.bias, a.bias_dtype, gc);
+      a.gate_out[(size_t)t * a.nH + head] = 1.0f / (1.0f + expf(-g));
+    }
     if (!is_q && slot < 0) return;
     T* dst = is_q ? (T*)a.q_out + (size_t)t * q_width + col
                   : (T*)a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.page_size + off) * d;
-    for (int p = threadIdx.x; p < half; p += blockDim.x) {
-      int i0, i1;
+    // pair p of the head with bias and rotation: elements i0, i1 and their values
+    auto pair = [&](int p, int& i0, int& i1, float& y0, float& y1) {
       const bool rotate = p < rot_half;
       if (rotate) {
         if (a.rope_style == 1) { i0 = p; i1 = p + rot_half; }
@@ -418,27 +442,56 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
         x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
         x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
       }
-      float y0 = x0, y1 = x1;
+      y0 = x0; y1 = x1;
       if (rotate) {
         const float cs = a.cs[(size_t)t * rot_half + p], sn = a.sn[(size_t)t * rot_half + p];
         y0 = x0 * cs - x1 * sn;
         y1 = x0 * sn + x1 * cs;
       }
-      dst[i0] = from_f<T>(y0);
-      dst[i1] = from_f<T>(y1);
+    };
+    float inv = 1.f;
+    if (a.unit_norm) {       // the head's sum of squares first (the block is one wave); the values are formed again below
+      float ss = 0.f;
+      for (int p = threadIdx.x; p < half; p += blockDim.x) {
+        int i0, i1;
+        float y0, y1;
+        pair(p, i0, i1, y0, y1);
+        ss += y0 * y0 + y1 * y1;
+      }
+      inv = rsqrtf(wave_sum(ss) / (float)d + a.norm_eps);
+    }
+    for (int p = threadIdx.x; p < half; p += blockDim.x) {
+      int i0, i1;
+      float y0, y1;
+      pair(p, i0, i1, y0, y1);
+      dst[i0] = from_f<T>(y0 * inv);
+      dst[i1] = from_f<T>(y1 * inv);
     }
   } else {
-    if (slot < 0) return;
     const int kh = head - a.nH - a.nKV;
+    if (kh >= a.nKV) return;
+    if (slot < 0 && !a.v_out) return;
     const int vcol = q_width + kv_width + kh * dv;              // value heads are dv wide
     T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * dv * a.page_size + off;
+    const T* vf = a.v_first ? (const T*)a.v_first + ((size_t)t * a.nKV + kh) * dv : nullptr;
+    T* vo = a.v_out ? (T*)a.v_out + ((size_t)t * a.nKV + kh) * dv : nullptr;
     for (int e = threadIdx.x; e < dv; e += 2 * blockDim.x) {    // two elements per thread and round: their loads go out together
       const int e1 = min(e + (int)blockDim.x, dv - 1);
       float x, x1;
       in2(vcol + e, vcol + e1, x, x1);
       if (a.bias) { x += load_dyn(a.bias, a.bias_dtype, vcol + e); x1 += load_dyn(a.bias, a.bias_dtype, vcol + e1); }
+      const bool second = e + (int)blockDim.x < dv;
+      if (vo) {
+        vo[e] = from_f<T>(x);
+        if (second) vo[e1] = from_f<T>(x1);
+      }
+      if (vf) {
+        x = (1.f - a.v_mix) * x + a.v_mix * to_f(vf[e]);
+        x1 = (1.f - a.v_mix) * x1 + a.v_mix * to_f(vf[e1]);
+      }
+      if (slot < 0) continue;
       vc[(size_t)e * a.page_size] = from_f<T>(x);
-      if (e + (int)blockDim.x < dv) vc[(size_t)e1 * a.page_size] = from_f<T>(x1);
+      if (second) vc[(size_t)e1 * a.page_size] = from_f<T>(x1);
     }
   }
 }
@@ -532,7 +585,8 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
 extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
                                const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
                                int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, int n_slices,
-                               long long slice_stride, int dv, void* stream) {
+                               long long slice_stride, int dv, int gate_cols, float* gate_out, int unit_norm, float norm_eps,
+                               const void* v_first, float v_mix, void* v_out, void* stream) {
   IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || slice_stride > 0), "rope_append: %d slices, %lld apart", n_slices, slice_stride);
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0 && dv > 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d dv=%d", T, nH, nKV, d, dv);
   IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
@@ -541,11 +595,14 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "rope_append: cache write without cache");
   IFX_REQUIRE(nH + 2 * nKV <= 65535, "rope_append: too many heads for one launch");
   if (T == 0) return 0;
+  IFX_REQUIRE(gate_cols == 0 || (gate_cols == nH && gate_out), "rope_append: %d gate columns for %d heads", gate_cols, nH);
+  IFX_REQUIRE(!(v_first || v_out) || nKV > 0, "rope_append: values to mix or to hand on, but no kv heads");
   RopeArgs a{qkv, n_slices, (size_t)slice_stride, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size,
-             q_out, k_cache, v_cache, dv};
+             q_out, k_cache, v_cache, dv, gate_cols, gate_out, unit_norm, norm_eps, v_first, v_mix, v_out};
+  const bool extras = gate_cols || unit_norm || v_first || v_out;
   hipStream_t s = (hipStream_t)stream;
   // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
-  if (dv == d && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
+  if (!extras && dv == d && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
       (!slots || page_size % 8 == 0)) {
     const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
     const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;
@@ -561,21 +618,21 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
 }
 
 // ---------------------------------------------------------------------------------------
-// out[t, i] = gate / (1 + exp(-gate)) * up, with gu[t] = [gate (I) | up (I)] or, interleaved,
+// out[t, i] = act(gate) * up (act: ACT_SILU gate / (1 + exp(-gate)), ACT_GELU_TANH the tanh form of gelu), with gu[t] = [gate (I) | up (I)] or, interleaved,
 // gu[t] = [gate_0, up_0, gate_1, up_1, ...].
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n, int interleaved) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n, int interleaved, int act) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const size_t t = idx / I;
   const int i = (int)(idx % I);
   const float g = to_f(gu[t * 2 * I + (interleaved ? 2 * i : i)]);
   const float u = to_f(gu[t * 2 * I + (interleaved ? 2 * i + 1 : I + i)]);
-  out[idx] = from_f<T>(g / (1.0f + expf(-g)) * u);
+  out[idx] = from_f<T>(gated_act(g, u, act));
 }
 
 // The interleaved bf16 case in 32-byte pieces: 8 gate/up pairs in, 8 results out (I a multiple of 8).
-__global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, size_t n8) {
+__global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, size_t n8, int act) {
   typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n8) return;
@@ -584,26 +641,27 @@ __global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* 
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const float g0 = (float)a[2 * e], u0 = (float)a[2 * e + 1], g1 = (float)b[2 * e], u1 = (float)b[2 * e + 1];
-    o[e] = (__bf16)(g0 / (1.0f + expf(-g0)) * u0);
-    o[e + 4] = (__bf16)(g1 / (1.0f + expf(-g1)) * u1);
+    o[e] = (__bf16)gated_act(g0, u0, act);
+    o[e + 4] = (__bf16)gated_act(g1, u1, act);
   }
   *(bf16x8*)(out + 8 * i) = o;
 }
 
-extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, void* stream) {
+extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, int act, void* stream) {
+  IFX_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "gated activation: unknown kind %d", act);
   IFX_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   const size_t n = (size_t)T * I;
   if (interleaved && dtype == DT_BF16 && I % 8 == 0) {
     const size_t n8 = n / 8;
     hipLaunchKernelGGL(swiglu_pairs_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const bf16_t*)gu, (bf16_t*)out, n8);
+                       (const bf16_t*)gu, (bf16_t*)out, n8, act);
     IFX_LAUNCH_CHECK();
   }
   const unsigned blocks = (unsigned)((n + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved);
-  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n, interleaved);
+  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved, act);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n, interleaved, act);
   else IFX_FAIL("swiglu: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

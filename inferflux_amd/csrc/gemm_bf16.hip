@@ -43,6 +43,7 @@ struct StreamOut {
   const bf16_t* norm_w;
   bf16_t* rows;
   float* pieces;
+  float mult;      // the product is multiplied by this before it is added (a model's factor on every sub-block's output)
 };
 
 // Sum over the four lanes col, col + 16, col + 32, col + 48, the same in all four.
@@ -187,7 +188,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
           bf16x2 y;
 #pragma unroll
           for (int r = 0; r < 2; ++r) {
-            v[r] = was[nt][q][r] + acc[nt][0][2 * q + r] * rs;
+            v[r] = was[nt][q][r] + acc[nt][0][2 * q + r] * rs * so.mult;
             y[r] = (__bf16)(v[r] * (float)nw[nt][q][r]);
             sq += v[r] * v[r];
           }
@@ -219,7 +220,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
         for (int r = 0; r < 4; r += 2) {
           const int n = n0 + 4 * g + r;  // even: gate at n, up at n + 1
           const float gt = acc[nt][mt][r] * rs, up = acc[nt][mt][r + 1] * rs;
-          if (4 * g + r < tile_rows && n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+          if (4 * g + r < tile_rows && n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gated_epilogue<EPI>(gt, up));
         }
       }
     }
@@ -316,8 +317,10 @@ static int launch(const void* x, const void* W, void* out, int out_dtype, int M,
     if constexpr (MT == 1) GO(float, 2);
     else IFX_FAIL("skinny_gemm: the stream epilogue takes at most 16 rows");
   } else if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+  else if (out_dtype == DT_BF16 && epi == 3) GO(bf16_t, 3);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
+  else if (epi == 3) GO(float, 3);
   else GO(float, 1);
 #undef GO
   IFX_LAUNCH_CHECK();
@@ -394,7 +397,7 @@ extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const v
 }
 
 // nt, waves, unroll = 0: chosen here from the shape.
-// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2].
+// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2]; epi 3: the same with the tanh form of gelu.
 // epi 2: the product is added to ``stream`` [M, N] (float, in place), rows_out [M, N] = bf16(stream * norm_w) and
 //        pieces_out [ceil(N / 16)][16] = sums of squares of the stream in runs of 16, for the norm that follows
 //        (M <= 16, N a multiple of 4, norm_w bfloat16 [N]); ``out`` is not used.
@@ -404,12 +407,12 @@ extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const v
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
                                int waves, int unroll, int epi, int tiled, const int* order, const float* scale_pieces,
                                int n_scale_pieces, float scale_width, float scale_eps, float* stream_io,
-                               const void* norm_w, void* rows_out, float* pieces_out, void* stream) {
+                               const void* norm_w, void* rows_out, float* pieces_out, float stream_mult, void* stream) {
   IFX_REQUIRE(tiled == 0 || tiled == 1 || (tiled >= 8 && tiled <= 16 && tiled % 2 == 0), "skinny_gemm: tiled=%d (0, 1, or 8 to 16 rows to a tile)", tiled);
   const int tile_rows = tiled >= 8 ? tiled : 16;
   IFX_REQUIRE((tiled && tile_rows == 16) || !order, "skinny_gemm: a tile order goes with a tiled copy of 16-row tiles");
   IFX_REQUIRE(epi == 0 || !order, "skinny_gemm: only the plain epilogue takes a tile order");
-  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0) || (epi == 2 && N % 4 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
+  IFX_REQUIRE(epi == 0 || ((epi == 1 || epi == 3) && N % 2 == 0) || (epi == 2 && N % 4 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
   IFX_REQUIRE(epi != 2 || (M <= 16 && stream_io && norm_w && rows_out && pieces_out),
               "skinny_gemm: the stream epilogue takes at most 16 rows (M=%d) and needs the stream, the norm's weight and two outputs", M);
   IFX_REQUIRE(!scale_pieces || (M <= 16 && n_scale_pieces > 0 && scale_width > 0.f),
@@ -462,7 +465,7 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   hipStream_t s = (hipStream_t)stream;
   const int k_tiles = ifx_tiled_cols(K) / 32;
   const RowScale scale{scale_pieces, n_scale_pieces, scale_width, scale_eps};
-  const StreamOut so{stream_io, (const bf16_t*)norm_w, (bf16_t*)rows_out, pieces_out};
+  const StreamOut so{stream_io, (const bf16_t*)norm_w, (bf16_t*)rows_out, pieces_out, stream_mult};
 #define CASE(MT_, NT_, U_)                                                                                             \
   if (mt == MT_ && nt == NT_ && unroll == U_)                                                                          \
     return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, tile_rows, s)  \
@@ -577,7 +580,7 @@ __global__ __launch_bounds__(256) void staged_gemm_kernel(const bf16_t* __restri
       for (int r = 0; r < 4; r += 2) {
         const int nn = n_base + 4 * g + r;  // even: gate at nn, up at nn + 1
         const float gt = acc[mt][r], up = acc[mt][r + 1];
-        if (nn + 1 < N) out[(size_t)m * (N / 2) + nn / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+        if (nn + 1 < N) out[(size_t)m * (N / 2) + nn / 2] = from_f<TO>(gated_epilogue<EPI>(gt, up));
       }
     }
   }
@@ -600,8 +603,10 @@ static int launch_staged(const void* x, const void* W, void* out, int out_dtype,
   hipLaunchKernelGGL((staged_gemm_kernel<MT, U, TO_, EPI_>), grid, dim3(256), 0, s, (const bf16_t*)x,         \
                      (const bf16_t*)W, (TO_*)out, part, M, N, K, cps)
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+  else if (out_dtype == DT_BF16 && epi == 3) GO(bf16_t, 3);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
+  else if (epi == 3) GO(float, 3);
   else GO(float, 1);
 #undef GO
   if (slices > 1) {
@@ -633,7 +638,7 @@ extern "C" int ifx_staged_gemm(const void* x, const void* W, void* out, int out_
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "staged_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "staged_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "staged_gemm: unknown out dtype %d", out_dtype);
-  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "staged_gemm: epilogue %d with N=%d", epi, N);
+  IFX_REQUIRE(epi == 0 || ((epi == 1 || epi == 3) && N % 2 == 0), "staged_gemm: epilogue %d with N=%d", epi, N);
   if (M == 0) return 0;
   const int mt = (M + 15) / 16;
   const int n_chunks = (K + KC - 1) / KC;

@@ -214,7 +214,7 @@ __global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVE
 #pragma unroll
       for (int r = 0; r < 4; r += 2) {   // even: gate at n0 + r, up at n0 + r + 1
         const float gt = acc[mt][r], up = acc[mt][r + 1];
-        v[r / 2] = gt / (1.0f + expf(-gt)) * up;
+        v[r / 2] = gated_epilogue<EPI>(gt, up);
       }
       if (whole) {
         store2(dst, v[0], v[1]);
@@ -294,8 +294,10 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
                      (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order, tile_rows, scale)
 #define GO_ALL(MINW_)                                    \
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0, MINW_); \
+  else if (out_dtype == DT_BF16 && epi == 3) GO(bf16_t, 3, MINW_); \
   else if (out_dtype == DT_BF16) GO(bf16_t, 1, MINW_);        \
   else if (epi == 0) GO(float, 0, MINW_);                     \
+  else if (epi == 3) GO(float, 3, MINW_);                     \
   else GO(float, 1, MINW_)
   if (waves >= MIN_WAVES) {
     GO_ALL(MIN_WAVES);
@@ -316,7 +318,8 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
 
 // x [M <= 128, K] times the tiled copy Wt of W [N, K], transposed.  ``waves``, ``slices``: as ifx_wide_gemm_plan
 // returned them; ``part``: slices * M * N floats when there is more than one slice.
-// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order).
+// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order); epi 3: the same
+// with the tanh form of gelu.
 // order: the row-tile order the copy was written with (or null); tile_rows: the rows to a tile it was written with.
 // ``out`` null with more than one slice: the partial sums are left in ``part`` for a kernel that adds them itself
 // (ifx_add_rmsnorm, ifx_rope_append).
@@ -330,7 +333,7 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   IFX_REQUIRE(M >= 0 && M <= MAX_ROWS && N > 0 && K > 0, "wide_gemm: M=%d must be at most %d (N=%d K=%d)", M, MAX_ROWS, N, K);
   IFX_REQUIRE(K % 8 == 0, "wide_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "wide_gemm: unknown out dtype %d", out_dtype);
-  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0 && !order && slices == 1), "wide_gemm: epilogue %d with N=%d, %d slices%s", epi, N,
+  IFX_REQUIRE(epi == 0 || ((epi == 1 || epi == 3) && N % 2 == 0 && !order && slices == 1), "wide_gemm: epilogue %d with N=%d, %d slices%s", epi, N,
               slices, order ? ", a tile order" : "");
   const int n_rounds = (K + WK - 1) / WK;
   IFX_REQUIRE(waves >= FEW_WAVES && waves <= MAX_WAVES && slices >= 1 && slices <= n_rounds, "wide_gemm: %d waves (%d-%d), %d slices of %d rounds",

@@ -1,0 +1,219 @@
+// A selective state-space mixer's kernels: the short causal convolution with its activation, and the scan.
+//
+// Both work on a step's flattened rows (requests end to end, a request's rows in position order) and carry
+// what a request needs from step to step in its state slot, one float32 row per slot:
+//   [C * (taps - 1)]  the convolution's last taps - 1 inputs, [channel][oldest ... newest]
+//   [C * N]           the recurrence's state S, [channel][state]
+// A request that starts finds its slot zeroed, which is "zeros before the start" for the convolution and S = 0.
+//
+//   convolution   u[t, c] = silu(b[c] + sum_j w[c, j] x[t - (taps - 1) + j, c]), the last column of w the current
+//                 token's; inputs before the step come from the slot, inputs before the request are zero.
+//   scan          dt = softplus(dt_raw[t, c] + dt_bias[c]);  S[c, n] <- exp(dt A[c, n]) S[c, n] + dt u[t, c] B[t, n];
+//                 y[t, c] = sum_n S[c, n] C[t, n] + D[c] u[t, c];  out[t, c] = y * silu(z[t, c]).
+//
+// Step sizes, decays, exponentials, the state and the sums are float whatever the activation type; u, B, C and z
+// come in the activation type.  A token's result depends on the tokens of its request before it and on nothing
+// else of the step: the order of the additions for (token, channel) is the same however the request was cut.
+#include "common.h"
+
+IFX_DEFINE_LAST_ERROR()
+
+#define MAX_TAPS 16
+
+struct ConvArgs {
+  const void* x;         // [T, ld] of the activation type; the convolution's channels are columns 0 .. C-1
+  int ld;
+  const void* w;         // [C, taps]
+  const void* b;         // [C] or null
+  int w_dtype;
+  float* state;          // [slots, state_stride]; the convolution's part starts at column 0
+  size_t state_stride;
+  const int* row_req;    // [T]
+  const int* q_start;    // [R]
+  const int* q_len;      // [R]
+  const int* slots;      // [R]
+  void* out;             // [T, C] of the activation type
+  int T, R, C, taps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
+  const int c = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+  if (c >= a.C) return;
+  const int r = a.row_req[t], t0 = a.q_start[r], i = t - t0, taps = a.taps;
+  const float* st = a.state + (size_t)a.slots[r] * a.state_stride + (size_t)c * (taps - 1);
+  const T* x = (const T*)a.x;
+  float acc = a.b ? load_dyn(a.b, a.w_dtype, c) : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = i - (taps - 1) + j;          // the input's place among the request's rows of this step
+    const float xv = src >= 0 ? to_f(x[(size_t)(t0 + src) * a.ld + c]) : st[src + taps - 1];
+    acc = fmaf(load_dyn(a.w, a.w_dtype, (size_t)c * taps + j), xv, acc);
+  }
+  ((T*)a.out)[(size_t)t * a.C + c] = from_f<T>(act_silu(acc));
+}
+
+// After the convolution has read the slots: every request's last taps - 1 inputs, from this step's rows and, where
+// the step brought fewer, from what the slot held.  One thread owns a (request, channel): it reads before it writes.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(ConvArgs a) {
+  const int c = blockIdx.x * 256 + threadIdx.x, r = blockIdx.y;
+  if (c >= a.C) return;
+  const int n = a.q_len[r], t0 = a.q_start[r], keep = a.taps - 1;
+  float* st = a.state + (size_t)a.slots[r] * a.state_stride + (size_t)c * keep;
+  const T* x = (const T*)a.x;
+  float v[MAX_TAPS - 1];
+#pragma unroll
+  for (int k = 0; k < MAX_TAPS - 1; ++k) {
+    if (k >= keep) break;
+    const int src = n - keep + k;
+    v[k] = src >= 0 ? to_f(x[(size_t)(t0 + src) * a.ld + c]) : st[k + n];
+  }
+#pragma unroll
+  for (int k = 0; k < MAX_TAPS - 1; ++k) {
+    if (k >= keep) break;
+    st[k] = v[k];
+  }
+}
+
+extern "C" int ifx_causal_conv(const void* x, int dtype, int ld, const void* w, const void* b, int w_dtype, float* state,
+                               long long state_stride, const int* row_req, const int* q_start, const int* q_len,
+                               const int* slots, void* out, int T, int R, int C, int taps, void* stream) {
+  IFX_REQUIRE(T >= 0 && R >= 0 && C > 0 && ld >= C, "causal_conv: bad sizes T=%d R=%d C=%d ld=%d", T, R, C, ld);
+  IFX_REQUIRE(taps >= 1 && taps <= MAX_TAPS, "causal_conv: %d taps outside 1..%d", taps, MAX_TAPS);
+  IFX_REQUIRE(state_stride >= (long long)C * (taps - 1), "causal_conv: a state row of %lld floats for %d x %d inputs", state_stride, C, taps - 1);
+  IFX_REQUIRE(T <= 65535 && R <= 65535, "causal_conv: too many rows for one launch");
+  if (T == 0 || R == 0) return 0;
+  ConvArgs a{x, ld, w, b, w_dtype, state, (size_t)state_stride, row_req, q_start, q_len, slots, out, T, R, C, taps};
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned cb = (unsigned)((C + 255) / 256);
+  if (dtype == DT_F32) {
+    hipLaunchKernelGGL(conv_silu_kernel<float>, dim3(cb, T), dim3(256), 0, s, a);
+    if (taps > 1) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(cb, R), dim3(256), 0, s, a);
+  } else if (dtype == DT_BF16) {
+    hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, dim3(cb, T), dim3(256), 0, s, a);
+    if (taps > 1) hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(cb, R), dim3(256), 0, s, a);
+  } else IFX_FAIL("causal_conv: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+struct ScanArgs {
+  const void* u;         // [T, C] the convolution's output
+  const float* dt_raw;   // [T, C] float: the step-size projection before bias and softplus
+  const void* dt_bias;   // [C]
+  const float* A;        // [C, N] float, negative
+  const void* bc;        // [T, ld_bc]: B in columns 0 .. N-1, C in columns N .. 2N-1
+  int ld_bc;
+  const void* D;         // [C]
+  int w_dtype;           // of dt_bias and D
+  const void* z;         // [T, ld_z] the gate's input, first column at z
+  int ld_z;
+  float* state;          // [slots, state_stride]; S starts at column state_offset
+  size_t state_stride, state_offset;
+  const int* q_start;
+  const int* q_len;
+  const int* slots;
+  void* out;             // [T, C]
+  int R, C, N;
+};
+
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// LANES lanes share a channel, each with NPT of its states (state n belongs to lane n / NPT); a token's sum over the
+// states is added across them in a fixed order.  TOK tokens' inputs are asked for together, so that the recurrence,
+// which is a chain from token to token, waits for memory once per TOK tokens.
+constexpr int LANES = 4, TOK = 4;
+
+template <typename T, int NPT>
+__global__ __launch_bounds__(256) void scan_kernel(ScanArgs a) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int c = idx / LANES, lg = idx % LANES, r = blockIdx.y;
+  if (c >= a.C) return;          // (C * LANES is a multiple of LANES: the lanes of a channel leave together)
+  const int N = a.N, n0 = lg * NPT;
+  const int t0 = a.q_start[r], n_tok = a.q_len[r];
+  float* S_mem = a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + (size_t)c * N + n0;
+  float S[NPT], An[NPT];
+#pragma unroll
+  for (int k = 0; k < NPT; ++k) {
+    const bool ok = n0 + k < N;
+    S[k] = ok ? S_mem[k] : 0.f;
+    An[k] = ok ? a.A[(size_t)c * N + n0 + k] : 0.f;
+  }
+  const float dtb = load_dyn(a.dt_bias, a.w_dtype, c), Dc = load_dyn(a.D, a.w_dtype, c);
+  const T* u = (const T*)a.u;
+  const T* bc = (const T*)a.bc;
+  const T* z = (const T*)a.z;
+  for (int i0 = 0; i0 < n_tok; i0 += TOK) {
+    float uv[TOK], dtv[TOK], zv[TOK], Bv[TOK][NPT], Cv[TOK][NPT];
+#pragma unroll
+    for (int q = 0; q < TOK; ++q) {
+      const bool live = i0 + q < n_tok;
+      const size_t t = (size_t)t0 + i0 + (live ? q : 0);
+      uv[q] = to_f(u[t * a.C + c]);
+      dtv[q] = a.dt_raw[t * a.C + c];
+      zv[q] = to_f(z[t * a.ld_z + c]);
+#pragma unroll
+      for (int k = 0; k < NPT; ++k) {
+        const int n = min(n0 + k, N - 1);
+        Bv[q][k] = to_f(bc[t * a.ld_bc + n]);
+        Cv[q][k] = to_f(bc[t * a.ld_bc + N + n]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < TOK; ++q) {
+      if (i0 + q >= n_tok) break;
+      const float dt = softplus_f(dtv[q] + dtb), dtu = dt * uv[q];
+      float y = 0.f;
+#pragma unroll
+      for (int k = 0; k < NPT; ++k) {
+        if (n0 + k < N) {
+          S[k] = fmaf(expf(dt * An[k]), S[k], dtu * Bv[q][k]);
+          y = fmaf(S[k], Cv[q][k], y);
+        }
+      }
+      y += __shfl_xor(y, 1, WAVE);      // the channel's four lanes are neighbours
+      y += __shfl_xor(y, 2, WAVE);
+      if (lg == 0) {
+        y = fmaf(Dc, uv[q], y);
+        ((T*)a.out)[((size_t)t0 + i0 + q) * a.C + c] = from_f<T>(y * act_silu(zv[q]));
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NPT; ++k)
+    if (n0 + k < N) S_mem[k] = S[k];
+}
+
+template <typename T>
+static int launch_scan(const ScanArgs& a, hipStream_t s) {
+  const int npt = (a.N + LANES - 1) / LANES;
+  const dim3 grid((unsigned)(((size_t)a.C * LANES + 255) / 256), a.R);
+#define GO(NPT_) hipLaunchKernelGGL((scan_kernel<T, NPT_>), grid, dim3(256), 0, s, a)
+  if (npt <= 1) GO(1);
+  else if (npt <= 2) GO(2);
+  else if (npt <= 4) GO(4);
+  else if (npt <= 6) GO(6);
+  else if (npt <= 8) GO(8);
+  else if (npt <= 12) GO(12);
+  else if (npt <= 16) GO(16);
+  else if (npt <= 32) GO(32);
+  else IFX_FAIL("selective_scan: %d states per channel (at most %d)", a.N, 32 * LANES);
+#undef GO
+  IFX_LAUNCH_CHECK();
+}
+
+extern "C" int ifx_selective_scan(const void* u, int dtype, const float* dt_raw, const void* dt_bias, const float* A,
+                                  const void* bc, int ld_bc, const void* D, int w_dtype, const void* z, int ld_z,
+                                  float* state, long long state_stride, long long state_offset, const int* q_start,
+                                  const int* q_len, const int* slots, void* out, int T, int R, int C, int N, void* stream) {
+  IFX_REQUIRE(T >= 0 && R >= 0 && C > 0 && N > 0, "selective_scan: bad sizes T=%d R=%d C=%d N=%d", T, R, C, N);
+  IFX_REQUIRE(ld_bc >= 2 * N && ld_z >= C, "selective_scan: rows of %d for B and C of %d, of %d for a gate of %d", ld_bc, N, ld_z, C);
+  IFX_REQUIRE(state_stride >= state_offset + (long long)C * N, "selective_scan: a state row of %lld floats for %lld + %d x %d", state_stride, state_offset, C, N);
+  IFX_REQUIRE(R <= 65535, "selective_scan: too many requests for one launch");
+  if (T == 0 || R == 0) return 0;
+  ScanArgs a{u, dt_raw, dt_bias, A, bc, ld_bc, D, w_dtype, z, ld_z, state, (size_t)state_stride, (size_t)state_offset,
+             q_start, q_len, slots, out, R, C, N};
+  if (dtype == DT_F32) return launch_scan<float>(a, (hipStream_t)stream);
+  if (dtype == DT_BF16) return launch_scan<bf16_t>(a, (hipStream_t)stream);
+  IFX_FAIL("selective_scan: unknown dtype %d", dtype);
+}

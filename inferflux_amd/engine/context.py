@@ -195,5 +195,14 @@ class StepContext:
             self._derived[key] = make()
         return self._derived[key]
 
+    def share(self, key, value) -> None:
+        """Leave ``value`` for the layers that run later in this step (``shared`` finds it): what one layer computes
+        for the step's rows and others mix in."""
+        self._derived[key] = value
+
+    def shared(self, key):
+        """What an earlier layer of this step left under ``key``, or None."""
+        return self._derived.get(key)
+
     def upload(self, array: np.ndarray) -> torch.Tensor:
         return torch.from_numpy(np.ascontiguousarray(array)).to(self.device)

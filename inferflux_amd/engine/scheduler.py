@@ -160,8 +160,8 @@ class Scheduler:
         for g, (k, pool) in enumerate(zip(need, self.manager.pools)):
             window = self.manager.groups[g].window
             if window is not None:   # a windowed group holds at most the window, a portion and two partial pages
-                P = self.manager.page_size
-                k = min(k, -(-(window + self.config.largest_portion) // P) + 2)
+                P = self.manager.page_size     # (and the pages of the first positions it keeps for good)
+                k = min(k, -(-(window + self.config.largest_portion) // P) + 2 + -(-self.manager.groups[g].keep_first // P))
             if k > pool.num_pages:
                 raise RequestRefused(f"request {rid!r} can never fit: {k} pages needed in cache group {g}, the pool has {pool.num_pages}")
         seq = Sequence_(rid, prompt, max_new, arrival=self._arrivals, n_prompt_original=len(prompt),

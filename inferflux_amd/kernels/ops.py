@@ -25,6 +25,8 @@ DT_F32, DT_BF16 = 0, 1
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
 
 ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
+ACT_SILU, ACT_GELU_TANH = 0, 1          # gated activations of a feed-forward: act(gate) * up
+_GATED_EPILOGUE = {ACT_SILU: 1, ACT_GELU_TANH: 3}    # ... as the epilogue number of the streaming products
 
 # The matrix-core attention module is compiled per head size, when a model with that head size
 # first runs; these sizes are compiled ahead by build_all().
@@ -55,6 +57,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("layernorm", ())
     yield ("latent", ())
     yield ("moe", ())
+    yield ("ssm", ())
     yield ("grouped_gemm", ())
     yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
@@ -122,19 +125,19 @@ def _call(mod: KernelModule, fname: str, argtypes, *args) -> None:
 
 
 # ----------------------------------------------------------------------------------------
-def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """float32 [T, H] rows of ``table`` [V, H] named by int32 ``ids`` [T] (ids are checked by the caller)."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] named by int32 ``ids`` [T] (ids are checked by the caller), times ``scale``."""
     _check(ids, "ids", (None,), torch.int32)
     _check(table, "table", (None, None))
     T, H = ids.shape[0], table.shape[1]
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
-    _call(load_module("core"), "ifx_embedding", (P, P, I, P, I, I, P),
-          ids.data_ptr(), table.data_ptr(), _dt(table), out.data_ptr(), T, H, _stream())
+    _call(load_module("core"), "ifx_embedding", (P, P, I, P, I, I, F, P),
+          ids.data_ptr(), table.data_ptr(), _dt(table), out.data_ptr(), T, H, float(scale), _stream())
     return out
 
 
-def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.Tensor, eps: float):
-    """``embedding`` for up to 16 tokens that also prepares the RMS norm (bfloat16 weight ``norm_weight`` [H]) which
+def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.Tensor, eps: float, scale: float = 1.0):
+    """``embedding`` (times ``scale``) for up to 16 tokens that also prepares the RMS norm (bfloat16 weight ``norm_weight`` [H]) which
     reads the stream first: returns (the float32 stream [T, H], that norm's rows up to the factor per row)."""
     _check(ids, "ids", (None,), torch.int32)
     _check(table, "table", (None, None))
@@ -145,15 +148,15 @@ def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     rows = torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
     pieces = torch.empty((-(-H // 4096), 16), dtype=torch.float32, device=table.device)
-    _call(load_module("core"), "ifx_embedding_norm", (P, P, I, P, P, P, P, I, I, P),
+    _call(load_module("core"), "ifx_embedding_norm", (P, P, I, P, P, P, P, I, I, F, P),
           ids.data_ptr(), table.data_ptr(), _dt(table), norm_weight.data_ptr(), out.data_ptr(), rows.data_ptr(),
-          pieces.data_ptr(), T, H, _stream())
+          pieces.data_ptr(), T, H, float(scale), _stream())
     return out, ScaledRows(rows, pieces, H, eps, norm_weight)
 
 
 def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``residual`` [T, H] float32 (+= ``delta`` in place when given and no ``rows``), then RMSNorm.
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta_scale: float = 1.0) -> torch.Tensor:
+    """``residual`` [T, H] float32 (+= ``delta_scale`` * ``delta`` in place when given and no ``rows``), then RMSNorm.
 
     With ``rows`` (int32 [R]) only those rows are normalised, into [R, H], and the residual is
     left untouched.
@@ -162,6 +165,8 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     T, H = residual.shape
     _check(weight, "weight", (H,))
     n_slices = 1
+    if isinstance(delta, ScaledDelta):             # a delta with its factor
+        delta, delta_scale = delta.value, delta_scale * delta.scale
     if isinstance(delta, SliceSums):               # partial sums: the kernel adds them in slice order
         _check(delta.parts, "delta", (None, T, H), torch.float32)
         n_slices, delta = delta.parts.shape[0], delta.parts
@@ -172,22 +177,22 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
         _check(rows, "rows", (None,), torch.int32)
         n = rows.shape[0]
     out = torch.empty((n, H), dtype=out_dtype, device=residual.device)
-    _call(load_module("core"), "ifx_add_rmsnorm", (P, P, I, P, I, P, I, P, I, I, F, I, I, LL, P),
+    _call(load_module("core"), "ifx_add_rmsnorm", (P, P, I, P, I, P, I, P, I, I, F, I, I, LL, F, P),
           residual.data_ptr(), _ptr(delta), _dt(delta) if delta is not None else 0, weight.data_ptr(),
           _dt(weight), out.data_ptr(), _DT[out_dtype], _ptr(rows), n, H, float(eps),
-          1 if (delta is not None and rows is None) else 0, n_slices, T * H, _stream())
+          1 if (delta is not None and rows is None) else 0, n_slices, T * H, float(delta_scale), _stream())
     return out
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
-    """cos and sin [T, pairs] of float(position) * inv_freq, computed in float."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0):
+    """``magnitude`` times cos and sin [T, pairs] of float(position) * inv_freq, computed in float."""
     _check(positions, "positions", (None,), torch.int32)
     _check(inv_freq, "inv_freq", (None,), torch.float32)
     T, n = positions.shape[0], inv_freq.shape[0]
     cs = torch.empty((T, n), dtype=torch.float32, device=positions.device)
     sn = torch.empty((T, n), dtype=torch.float32, device=positions.device)
-    _call(load_module("core"), "ifx_rope_table", (P, P, P, P, I, I, P),
-          positions.data_ptr(), inv_freq.data_ptr(), cs.data_ptr(), sn.data_ptr(), T, n, _stream())
+    _call(load_module("core"), "ifx_rope_table", (P, P, P, P, I, I, F, P),
+          positions.data_ptr(), inv_freq.data_ptr(), cs.data_ptr(), sn.data_ptr(), T, n, float(magnitude), _stream())
     return cs, sn
 
 
@@ -195,8 +200,14 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rope_style: int,
                 rotary_dim: int, n_heads: int, n_kv_heads: int, head_dim: int,
                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int,
-                v_head_dim: Optional[int] = None) -> torch.Tensor:
+                v_head_dim: Optional[int] = None, unit_norm_eps: Optional[float] = None, gate_out: Optional[torch.Tensor] = None,
+                v_first: Optional[torch.Tensor] = None, v_mix: float = 0.0, v_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Bias, rotation and cache write of one step's projections; returns q [T, n_heads, head_dim].
+
+    Optionally: ``unit_norm_eps`` divides every q and k head by its root mean square (eps inside the root) after the
+    rotation; ``gate_out`` (float32 [T, n_heads]) receives sigmoid(x + bias) of n_heads further columns behind q, k and v
+    (a gate per head on the attention's output); ``v_first`` [T, n_kv_heads v_head_dim] is mixed into the values before
+    they are cached, v <- (1 - v_mix) v + v_mix v_first; ``v_out`` receives the values as projected, before any mixing.
 
     ``qkv`` is [T, (n_heads + n_kv_heads) head_dim + n_kv_heads v_head_dim] when the keys and values are
     written (``slots`` int32 [T] = page * page_size + offset; ``v_head_dim`` None: as wide as the keys), or
@@ -205,7 +216,8 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     """
     T = qkv.shape[0]
     dv = head_dim if v_head_dim is None else int(v_head_dim)
-    width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * dv
+    gate_cols = n_heads if gate_out is not None else 0
+    width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * dv + gate_cols
     n_slices = 1
     if isinstance(qkv, SliceSums):                  # partial sums: the kernel adds them in slice order
         _check(qkv.parts, "qkv", (None, T, width), torch.float32)
@@ -224,29 +236,39 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
         _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, dv, page_size), dtype)
     elif n_kv_heads != 0:
         raise KernelError("rope_append: keys and values given but no slots to write them to")
+    if gate_out is not None:
+        _check(gate_out, "gate_out", (T, n_heads), torch.float32)
+    for t, nm in ((v_first, "v_first"), (v_out, "v_out")):
+        if t is not None:
+            _check(t, nm, (T, n_kv_heads * dv), dtype)
     q = torch.empty((T, n_heads, head_dim), dtype=dtype, device=qkv.device)
-    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, I, P),
+    _call(load_module("core"), "ifx_rope_append",
+          (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, I, I, P, I, F, P, F, P, P),
           qkv.data_ptr(), _DT[dtype], _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
           _ptr(cos) if rope_style != ROPE_NONE else 0, _ptr(sin) if rope_style != ROPE_NONE else 0, rope_style,
           rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache),
-          n_slices, T * width, dv, _stream())
+          n_slices, T * width, dv, gate_cols, _ptr(gate_out), 1 if unit_norm_eps is not None else 0,
+          float(unit_norm_eps or 0.0), _ptr(v_first), float(v_mix), _ptr(v_out), _stream())
     return q
 
 
-def swiglu(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
-    """silu(gate) * up [T, I] from [T, 2I] laid out [gate | up] or, interleaved, gate_0, up_0, gate_1, ..."""
+def swiglu(gate_up: torch.Tensor, interleaved: bool = False, act: int = ACT_SILU) -> torch.Tensor:
+    """act(gate) * up [T, I] from [T, 2I] laid out [gate | up] or, interleaved, gate_0, up_0, gate_1, ...; ``act``:
+    ACT_SILU (the default) or ACT_GELU_TANH."""
     _check(gate_up, "gate_up", (None, None))
     T, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError("swiglu: odd width")
     out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
-    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, P),
-          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, _stream())
+    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, I, P),
+          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, int(act), _stream())
     return out
 
 
 def _delta_args(delta, shape, name):
     """(pointer, dtype code, slices, elements between slices) of a tensor or of a product left as ``SliceSums``."""
+    if isinstance(delta, ScaledDelta):
+        delta = delta.tensor()
     if isinstance(delta, SliceSums):
         _check(delta.parts, name, (None, *shape), torch.float32)
         return delta.parts.data_ptr(), DT_F32, delta.parts.shape[0], delta.parts[0].numel()
@@ -634,6 +656,25 @@ class ScaledRows:
         return self.rows.dtype
 
 
+class ScaledDelta:
+    """A sub-block's output that is added to the stream times ``scale`` (a model's factor on every sub-block's output):
+    ``value`` is a tensor or ``SliceSums``.  ``add_rmsnorm`` takes it as its delta; ``tensor()`` forms it for everyone
+    else."""
+
+    __slots__ = ("value", "scale")
+
+    def __init__(self, value, scale: float):
+        self.value, self.scale = value, float(scale)
+
+    @property
+    def shape(self):
+        return self.value.shape
+
+    def tensor(self) -> torch.Tensor:
+        v = self.value.sum(torch.float32) if isinstance(self.value, SliceSums) else self.value.float()
+        return v * self.scale
+
+
 class SliceSums:
     """A product left as partial sums over slices of K: it stands for ``parts.sum(0)`` (float32 [S, M, N], added in
     slice order).  ``add_rmsnorm`` takes it as its delta and ``rope_append`` as its q/k/v, which saves the kernel
@@ -688,8 +729,8 @@ def adds_into_stream(n_rows: int, weight, norm_weight: torch.Tensor) -> bool:
 
 
 def linear_into_stream(x: torch.Tensor, weight: LinearWeight, stream: torch.Tensor, norm_weight: torch.Tensor,
-                       eps: float) -> ScaledRows:
-    """``stream`` [M <= 16, N] (float32) += x [M, K] W^T in place, as the product's epilogue, which also prepares
+                       eps: float, mult: float = 1.0) -> ScaledRows:
+    """``stream`` [M <= 16, N] (float32) += ``mult`` * x [M, K] W^T in place, as the product's epilogue, which also prepares
     the RMS norm that follows (weight ``norm_weight`` [N] bfloat16): returns its rows up to the factor per row."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
@@ -704,11 +745,11 @@ def linear_into_stream(x: torch.Tensor, weight: LinearWeight, stream: torch.Tens
     w = weight.rows if weight.tiled is None else weight.tiled
     _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
           x.data_ptr(), w.data_ptr(), 0, DT_F32, M, N, K, 0, 0, 0, 2, 0 if weight.tiled is None else tile_rows, 0,
-          0, 0, 0.0, 0.0, stream.data_ptr(), norm_weight.data_ptr(), rows.data_ptr(), pieces.data_ptr(), _stream())
+          0, 0, 0.0, 0.0, stream.data_ptr(), norm_weight.data_ptr(), rows.data_ptr(), pieces.data_ptr(), float(mult), _stream())
     return ScaledRows(rows, pieces, N, eps, norm_weight)
 
 
-_SKINNY_ARGS = (P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, F, F, P, P, P, P, P)
+_SKINNY_ARGS = (P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, F, F, P, P, P, P, F, P)
 
 
 def pair_tile_order(n_heads: int, head_dim: int) -> list:
@@ -754,11 +795,12 @@ def qkv_rope_append(x: torch.Tensor, weight: LinearWeight, bias: Optional[torch.
 
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False,
-                tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None, tile_rows: int = 16) -> torch.Tensor:
+                tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None, tile_rows: int = 16,
+                act: int = ACT_SILU) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
     accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
-    With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2].
-    With ``tiled`` (``tile_weights(weight, order, tile_rows)``) the kernel streams that copy instead of the rows.
+    With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is act(gate) * up [M, N/2] (``act``:
+    ACT_SILU or ACT_GELU_TANH).  With ``tiled`` (``tile_weights(weight, order, tile_rows)``) the kernel streams that copy instead of the rows.
     ``x`` may be ``ScaledRows``."""
     x, scale = _scale_args(x)
     _check(x, "x", (None, None), torch.bfloat16)
@@ -778,12 +820,13 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         raise KernelError("skinny_gemm: a tile order goes with a tiled copy and a plain product")
     _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
           x.data_ptr(), (weight if tiled is None else tiled).data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves,
-          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else tile_rows, _ptr(order), *scale, 0, 0, 0, 0, _stream())
+          unroll, _GATED_EPILOGUE[act] if swiglu_pairs else 0, 0 if tiled is None else tile_rows, _ptr(order), *scale, 0, 0, 0, 0,
+          1.0, _stream())
     return out
 
 
 def wide_gemm(x, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
-              slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False):
+              slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False, act: int = ACT_SILU):
     """bfloat16 x [M <= 128, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
     of a workgroup: the product for 17-64 rows, for 65-128 rows of weights with few rows, and for 9-16 rows of large
     tall weights.  ``waves`` (4-16 per workgroup, 8 beyond 64 rows; one tile of weight rows each) and ``slices`` of K
@@ -809,12 +852,12 @@ def wide_gemm(x, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, 
     out = None if keep else torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
     _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, I, P, I, F, F, P),
           x.data_ptr(), weight.tiled.data_ptr(), _ptr(out), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
-          1 if swiglu_pairs else 0, _ptr(weight.order), weight.tile_rows, *scale, _stream())
+          _GATED_EPILOGUE[act] if swiglu_pairs else 0, _ptr(weight.order), weight.tile_rows, *scale, _stream())
     return SliceSums(part, out_dtype) if keep else out
 
 
 def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                slices: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
+                slices: int = 0, unroll: int = 0, swiglu_pairs: bool = False, act: int = ACT_SILU) -> torch.Tensor:
     """The same product as skinny_gemm with x staged in LDS and shared by the waves of a workgroup
     (64 weight rows per workgroup, K cut into ``slices``; 0 lets the kernel choose)."""
     _check(x, "x", (None, None), torch.bfloat16)
@@ -831,7 +874,7 @@ def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
     _call(mod, "ifx_staged_gemm", (P, P, P, I, P, I, I, I, I, I, I, P),
           x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], _ptr(part), M, N, K, slices, unroll,
-          1 if swiglu_pairs else 0, _stream())
+          _GATED_EPILOGUE[act] if swiglu_pairs else 0, _stream())
     return out
 
 
@@ -971,9 +1014,9 @@ def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional
     return None
 
 
-def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) where ``weight_pairs`` [2I, K] (a tensor or a ``LinearWeight``) alternates the
-    rows of Wg and Wu.  For few rows the activation is the product's epilogue; otherwise a second kernel
+def linear_swiglu(x: torch.Tensor, weight_pairs, act: int = ACT_SILU) -> torch.Tensor:
+    """act(x Wg^T) * (x Wu^T) (``act``: ACT_SILU or ACT_GELU_TANH) where ``weight_pairs`` [2I, K] (a tensor or a
+    ``LinearWeight``) alternates the rows of Wg and Wu.  For few rows the activation is the product's epilogue; otherwise a second kernel
     applies it."""
     M, K = x.shape
     if isinstance(x, ScaledRows) and not takes_scaled_rows(M, weight_pairs):
@@ -985,20 +1028,23 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
     if rows.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
         kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":
-            return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled, tile_rows=tile_rows)
+            return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled, tile_rows=tile_rows, act=act)
         if kind == "wide":
-            return wide_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
+            return wide_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True, act=act)
         if kind == "staged":
-            return staged_gemm(x, rows, torch.bfloat16, swiglu_pairs=True)
-    return swiglu(linear(x, rows), interleaved=True)
+            return staged_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, act=act)
+    return swiglu(linear(x, rows), interleaved=True, act=act)
 
 
 # ----------------------------------------------------------------------------------------
 def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor,
                     positions: torch.Tensor, block_table: torch.Tensor, window: Optional[int],
-                    scale: float) -> torch.Tensor:
+                    scale: float, keep_first: int = 0, sink: Optional[float] = None,
+                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal (optionally windowed) attention of q [T, nH, d] over the paged cache (K [pages, nKV, page, d],
-    V [pages, nKV, dv, page]; dv may differ from d); returns [T, nH*dv]."""
+    V [pages, nKV, dv, page]; dv may differ from d); returns [T, nH*dv].  ``keep_first``: a windowed query also sees
+    the first so many positions of its request; ``sink``: the score of a key without value that is added to the
+    softmax's denominator (None: no such key); ``gate`` float32 [T, nH]: a factor on every head's output."""
     _check(q, "q", (None, None, None))
     T, nH, d = q.shape
     _check(k_cache, "k_cache", (None, None, None, d), q.dtype)
@@ -1008,11 +1054,69 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _check(row_req, "row_req", (T,), torch.int32)
     _check(positions, "positions", (T,), torch.int32)
     _check(block_table, "block_table", (None, None), torch.int32)
+    if gate is not None:
+        _check(gate, "gate", (T, nH), torch.float32)
     out = torch.empty((T, nH * dv), dtype=q.dtype, device=q.device)
-    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P),
+    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, P, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, dv, page_size,
-          int(window or 0), float(scale), _stream())
+          int(window or 0), float(scale), int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate), _stream())
+    return out
+
+
+# ----------------------------------------------------------------------------------------
+def causal_conv_silu(x: torch.Tensor, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                     row_req: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """silu of a causal convolution per channel over each request's rows: the first ``channels`` columns of ``x``
+    [T, >= channels] with ``weight`` [channels, taps] (the last column is the current token's) and ``bias``.  A request's
+    last taps - 1 inputs live in the first channels * (taps - 1) floats of its row of ``state`` [slots, n] (float32,
+    zero for a request that starts), are read as the inputs before this step's and replaced by this step's last.
+    ``row_req`` [T], ``q_start`` / ``q_len`` / ``slots`` [R] (int32) describe the step.  Returns [T, channels]."""
+    _check(x, "x", (None, None))
+    T, ld = x.shape
+    _check(weight, "weight", (channels, None))
+    taps = weight.shape[1]
+    if bias is not None:
+        _check(bias, "bias", (channels,), weight.dtype)
+    _check(state, "state", (None, None), torch.float32)
+    _check(row_req, "row_req", (T,), torch.int32)
+    R = q_start.shape[0]
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _check(t, nm, (R,), torch.int32)
+    out = torch.empty((T, channels), dtype=x.dtype, device=x.device)
+    _call(load_module("ssm"), "ifx_causal_conv", (P, I, I, P, P, I, P, LL, P, P, P, P, P, I, I, I, I, P),
+          x.data_ptr(), _dt(x), ld, weight.data_ptr(), _ptr(bias), _dt(weight), state.data_ptr(), state.shape[1],
+          row_req.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, channels, taps, _stream())
+    return out
+
+
+def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, bc: torch.Tensor,
+                   D: torch.Tensor, z: torch.Tensor, state: torch.Tensor, state_offset: int, q_start: torch.Tensor,
+                   q_len: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """The recurrence of a selective state-space mixer over each request's rows, then the gate:
+    dt = softplus(dt_raw + dt_bias); S[c, n] <- exp(dt A[c, n]) S[c, n] + dt u[c] B[n]; y[c] = sum_n S[c, n] C[n] + D[c] u[c];
+    out = y * silu(z).  ``u`` [T, C], ``dt_raw`` float32 [T, C], ``A`` float32 [C, N] (negative), ``bc`` [T, >= 2N] with B
+    then C, ``z`` a view [T, C] of rows that may be wider (its row stride is taken), ``state`` float32 [slots, n] with a
+    request's S at ``state_offset`` of its row.  All of the recurrence is float.  Returns [T, C] in u's type."""
+    _check(u, "u", (None, None))
+    T, C = u.shape
+    _check(dt_raw, "dt_raw", (T, C), torch.float32)
+    _check(A, "A", (C, None), torch.float32)
+    N = A.shape[1]
+    _check(dt_bias, "dt_bias", (C,))
+    _check(D, "D", (C,), dt_bias.dtype)
+    _check(bc, "bc", (T, None), u.dtype)
+    if not (isinstance(z, torch.Tensor) and z.is_cuda and z.dtype == u.dtype and tuple(z.shape) == (T, C) and z.stride(1) == 1):
+        raise KernelError("selective_scan: z must be a [T, C] view with contiguous rows in u's type")
+    _check(state, "state", (None, None), torch.float32)
+    R = q_start.shape[0]
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _check(t, nm, (R,), torch.int32)
+    out = torch.empty((T, C), dtype=u.dtype, device=u.device)
+    _call(load_module("ssm"), "ifx_selective_scan", (P, I, P, P, P, P, I, P, I, P, I, P, LL, LL, P, P, P, P, I, I, I, I, P),
+          u.data_ptr(), _dt(u), dt_raw.data_ptr(), dt_bias.data_ptr(), A.data_ptr(), bc.data_ptr(), bc.shape[1], D.data_ptr(),
+          _dt(D), z.data_ptr(), z.stride(0) if T else C, state.data_ptr(), state.shape[1], int(state_offset), q_start.data_ptr(),
+          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, C, N, _stream())
     return out
 
 

@@ -11,6 +11,21 @@ activation type first and adds the bias afterwards, cuda_kernels.cu:518-527).
 
 An execution that reads another entry's cache (binding.writes_cache False) projects and
 encodes only its queries.
+
+Optional mechanisms, each a constructor argument that is off by default:
+  ``keep_first``      a windowed query at position i also sees the request's first ``keep_first`` positions, at their true
+                      places: j <= i and (i - j < window or j < keep_first); the cache keeps their pages.
+  ``sink``            a key without value with this score joins the softmax's denominator: p_j = exp(s_j) /
+                      (exp(sink) + sum_j exp(s_j)); with 0 that is "one added to the denominator".
+  ``unit_norm_eps``   after the rotation every q and k head is divided by its root mean square (eps inside the root; an
+                      RMS norm without weight).
+  ``output_gate``     head h's output is multiplied by sigmoid(W_g x)_h before the output projection (W_g [heads, H], a
+                      further block of rows of the fused projection).
+  ``value_mix``       "source": this layer hands the step's values (as projected) on to the layers after it; "mix": this
+                      layer caches v <- (1 - lambda) v + lambda v_source instead of its own, lambda a scalar tensor.  The
+                      layers must agree in kv heads and value width.
+  ``tensors``         full names of the tensors in the model file ("q", "k", "v", "o", "q_bias", "k_bias", "v_bias", "gate",
+                      "mix") where they are not ``<name>.q_proj.weight`` and so on.
 """
 from __future__ import annotations
 
@@ -32,7 +47,9 @@ class PagedAttention(Mixer):
 
     def __init__(self, name: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, bias: bool = True, window: Optional[int] = None,
-                 scale: Optional[float] = None, init_std: float = 0.02, v_head_dim: Optional[int] = None):
+                 scale: Optional[float] = None, init_std: float = 0.02, v_head_dim: Optional[int] = None,
+                 keep_first: int = 0, sink: Optional[float] = None, unit_norm_eps: Optional[float] = None,
+                 output_gate: bool = False, value_mix: Optional[str] = None, tensors: Optional[Mapping[str, str]] = None):
         """``v_head_dim``: the width of a value head where it differs from ``head_dim`` (such a layer runs on the
         kernels that take both widths: the plain attention kernel and the unfused projection path)."""
         if n_heads % n_kv_heads:
@@ -43,32 +60,57 @@ class PagedAttention(Mixer):
         self.bias, self.window, self.init_std = bool(bias), (int(window) if window else None), init_std
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = build_part("position", position)
+        self.keep_first = max(int(keep_first or 0), 0) if self.window else 0
+        self.sink = None if sink is None else float(sink)
+        self.unit_norm_eps = None if unit_norm_eps is None else float(unit_norm_eps)
+        self.output_gate = bool(output_gate)
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError(f"{name}: value_mix '{value_mix}' unknown (None, 'source' or 'mix')")
+        self.value_mix, self.mix_weight = value_mix, 0.0
+        self.names = {"q": f"{name}.q_proj.weight", "k": f"{name}.k_proj.weight", "v": f"{name}.v_proj.weight",
+                      "o": f"{name}.o_proj.weight", "q_bias": f"{name}.q_proj.bias", "k_bias": f"{name}.k_proj.bias",
+                      "v_bias": f"{name}.v_proj.bias", "gate": f"{name}.gate.weight", "mix": f"{name}.value_mix"}
+        self.names.update(tensors or {})
+        # (what the kernels fused for the plain case do not do: then the projection, the row kernel and attention run one by one)
+        self._extras = self.unit_norm_eps is not None or self.output_gate or self.value_mix is not None
         self.w_qkv = self.b_qkv = self.w_o = self._w_q = None
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(self.n_kv_heads, self.head_dim, self.window,
-                         self.v_head_dim if self.v_head_dim != self.head_dim else None)
+                         self.v_head_dim if self.v_head_dim != self.head_dim else None, self.keep_first)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         H, d, dv, s = self.hidden_size, self.head_dim, self.v_head_dim, ("normal", self.init_std)
+        nm = self.names
         out = {
-            f"{self.name}.q_proj.weight": ParamSpec((self.n_heads * d, H), s),
-            f"{self.name}.k_proj.weight": ParamSpec((self.n_kv_heads * d, H), s),
-            f"{self.name}.v_proj.weight": ParamSpec((self.n_kv_heads * dv, H), s),
-            f"{self.name}.o_proj.weight": ParamSpec((H, self.n_heads * dv), s),
+            nm["q"]: ParamSpec((self.n_heads * d, H), s),
+            nm["k"]: ParamSpec((self.n_kv_heads * d, H), s),
+            nm["v"]: ParamSpec((self.n_kv_heads * dv, H), s),
+            nm["o"]: ParamSpec((H, self.n_heads * dv), s),
         }
         if self.bias:
-            out[f"{self.name}.q_proj.bias"] = ParamSpec((self.n_heads * d,), s)
-            out[f"{self.name}.k_proj.bias"] = ParamSpec((self.n_kv_heads * d,), s)
-            out[f"{self.name}.v_proj.bias"] = ParamSpec((self.n_kv_heads * dv,), s)
+            out[nm["q_bias"]] = ParamSpec((self.n_heads * d,), s)
+            out[nm["k_bias"]] = ParamSpec((self.n_kv_heads * d,), s)
+            out[nm["v_bias"]] = ParamSpec((self.n_kv_heads * dv,), s)
+        if self.output_gate:
+            out[nm["gate"]] = ParamSpec((self.n_heads, H), s)
+        if self.value_mix is not None:       # (the source layer's tensor is in the file too; nothing reads it)
+            out[nm["mix"]] = ParamSpec((), ("uniform", 0.2, 0.8))
         return out
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        n = self.name
-        self.w_qkv = self._prepare_qkv(concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"]),
-                                       self.n_heads + 2 * self.n_kv_heads)
-        self.b_qkv = concat_weights([tensors[f"{n}.{p}_proj.bias"] for p in "qkv"]) if self.bias else None
-        self.w_o = ops.prepare_linear(tensors[f"{n}.o_proj.weight"])
+        nm = self.names
+        blocks = [tensors[nm[p]] for p in "qkv"] + ([tensors[nm["gate"]]] if self.output_gate else [])
+        self.w_qkv = self._prepare_qkv(concat_weights(blocks), self.n_heads + 2 * self.n_kv_heads)
+        self.b_qkv = None
+        if self.bias:
+            biases = [tensors[nm[p + "_bias"]] for p in "qkv"]
+            if self.output_gate:
+                biases.append(torch.zeros(self.n_heads, dtype=biases[0].dtype, device=biases[0].device))
+            self.b_qkv = concat_weights(biases)
+        self.w_o = ops.prepare_linear(tensors[nm["o"]])
+        if self.value_mix == "mix":
+            self.mix_weight = float(tensors[nm["mix"]].float().item())
         self._w_q = None
 
     def _prepare_qkv(self, weight: torch.Tensor, heads: int):
@@ -76,7 +118,8 @@ class PagedAttention(Mixer):
         row tiles are ordered so that the fused projection + rotation kernel finds both halves of a rotation
         pair in one lane (plain products read the same copy through the order)."""
         order = None
-        if self.head_dim % 32 == 0 and self.v_head_dim == self.head_dim and weight.is_cuda and weight.dtype == torch.bfloat16:
+        if (self.head_dim % 32 == 0 and self.v_head_dim == self.head_dim and weight.is_cuda and weight.dtype == torch.bfloat16
+                and not self._extras):
             order = torch.tensor(ops.pair_tile_order(heads, self.head_dim), dtype=torch.int32, device=weight.device)
         return ops.prepare_linear(weight, order)
 
@@ -87,10 +130,46 @@ class PagedAttention(Mixer):
 
     def _project_out(self, out, sink):
         if sink is not None and ops.adds_into_stream(out.shape[0], self.w_o, sink.norm_weight):
-            return ops.linear_into_stream(out, self.w_o, sink.stream, sink.norm_weight, sink.eps)
+            return ops.linear_into_stream(out, self.w_o, sink.stream, sink.norm_weight, sink.eps, sink.mult)
         return ops.linear(out, self.w_o, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself
 
+    def _attend(self, q, cache, ctx, gate=None):
+        return paged_attention(q, cache, ctx, self.window, self.scale, self.keep_first, self.sink, gate)
+
+    def _forward_extras(self, h, ctx, binding: MixerBinding, sink):
+        """The step with the optional mechanisms: the fused projection (with the gate's rows), one row kernel for bias,
+        rotation, unit norms, value mixing and the cache write, attention with the gate as a factor on its output."""
+        if not binding.writes_cache:
+            raise ValueError(f"{self.name}: a layer with unit norms, an output gate or value mixing owns its cache")
+        cache, nH, nKV, d, dv, T = binding.cache, self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim, h.shape[0]
+        style, rotary_dim, cos, sin = self.position.kernel_args(ctx)
+        if self.position.needs_apply:
+            raise ValueError(f"{self.name}: these mechanisms need a position part that gives the kernels a rotation table")
+        t = ctx.timer
+        qkv = ops.linear(h, self.w_qkv, keep_slices=True)
+        dtype = qkv.dtype
+        gate = torch.empty((T, nH), dtype=torch.float32, device=ctx.device) if self.output_gate else None
+        key = ("value_mix", nKV, dv)
+        v_first = v_out = None
+        if self.value_mix == "source":
+            v_out = torch.empty((T, nKV * dv), dtype=dtype, device=ctx.device)
+            ctx.share(key, v_out)
+        elif self.value_mix == "mix":
+            v_first = ctx.shared(key)
+            if v_first is None:
+                raise ValueError(f"{self.name}: mixes in the values of an earlier layer, but none has handed any on in this step")
+        q = ops.rope_append(qkv, self.b_qkv, ctx.write_slots(cache.group), cos, sin, style, rotary_dim, nH, nKV, d, cache.k, cache.v,
+                            cache.page_size, dv, self.unit_norm_eps, gate, v_first, self.mix_weight, v_out)
+        if t is not None:
+            t.mark("mixer.qkv")
+        a = self._attend(q, cache, ctx, gate)
+        if t is not None:
+            t.mark("mixer.attention")
+        return self._project_out(a, sink)
+
     def forward(self, h, ctx, binding: MixerBinding, sink=None):
+        if self._extras:
+            return self._forward_extras(h, ctx, binding, sink)
         cache = binding.cache
         nH, d = self.n_heads, self.head_dim
         nKV = self.n_kv_heads if binding.writes_cache else 0
@@ -110,7 +189,7 @@ class PagedAttention(Mixer):
                                     cache.v if slots is not None else None, cache.page_size)
             if t is not None:
                 t.mark("mixer.qkv")
-            a = paged_attention(q, cache, ctx, self.window, self.scale)
+            a = self._attend(q, cache, ctx)
             if t is not None:
                 t.mark("mixer.attention")
             return self._project_out(a, sink)
@@ -122,7 +201,7 @@ class PagedAttention(Mixer):
                             cache.page_size, self.v_head_dim)
         if t is not None:
             t.mark("mixer.qkv")
-        a = paged_attention(q, cache, ctx, self.window, self.scale)
+        a = self._attend(q, cache, ctx)
         if t is not None:
             t.mark("mixer.attention")
         return self._project_out(a, sink)

@@ -131,10 +131,12 @@ class MixerBinding:
 @dataclasses.dataclass
 class StreamSink:
     """Where a mixer or feed-forward may add its result itself: the float32 stream, and the weight and eps
-    of the RMS norm that reads the stream next."""
+    of the RMS norm that reads the stream next.  ``mult`` is the factor on what is added (a model's factor on every
+    sub-block's output; 1 otherwise)."""
     stream: torch.Tensor
     norm_weight: torch.Tensor
     eps: float
+    mult: float = 1.0
 
 
 class Mixer(Part):

@@ -6,6 +6,9 @@
 delta, and the norm that follows adds it to the float32 stream in the same kernel that
 normalises (the reference's ResidualAddRmsNorm, cuda_kernels.cu:617-671).
 
+With ``residual_scale`` m the adds are x <- x + m * sub-block(norm(x)) (the deltas are handed on with their factor,
+``ScaledDelta``), and a layer may have no feed-forward (then no second norm either).
+
 "outnorm" puts the norms on the sub-blocks' outputs instead: x <- x + norm1(mixer(x)), then
 x <- x + norm2(ffn(x)); the sub-blocks read the stream itself (rounded to the activation type), and a layer may
 have no feed-forward.  Its norms are parts with ``add_to(stream, delta, cast_dtype)``, which adds the normed delta
@@ -21,7 +24,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from ..kernels.ops import ScaledRows
+from ..kernels.ops import ScaledDelta, ScaledRows
 from .base import Block, MixerBinding, StreamSink, build_part, register_part
 from .plan import LayerSpec
 
@@ -40,49 +43,61 @@ def normed_for(norm, reader, residual, pending, ctx):
     return norm.forward(residual, pending, ctx.act_dtype)
 
 
-def _sink(part, residual, norm):
+def _sink(part, residual, norm, mult=1.0):
     if norm is None or not getattr(part, "adds_to_stream", False):
         return None
     params = norm.rms_params()
-    return StreamSink(residual, *params) if params is not None else None
+    return StreamSink(residual, *params, mult) if params is not None else None
 
 
 @register_part("block", "prenorm")
 class PreNormBlock(Block):
     graph_safe = True
 
-    def __init__(self, layer: LayerSpec, hidden_size: int):
-        if layer.norm_in is None or layer.norm_post is None or layer.ffn is None or layer.extra:
-            raise ValueError(f"layer {layer.prefix}: the prenorm block is two norms, a mixer and a feed-forward, no more and no less")
+    def __init__(self, layer: LayerSpec, hidden_size: int, residual_scale: float = 1.0):
+        if layer.norm_in is None or layer.extra or (layer.ffn is None) != (layer.norm_post is None):
+            raise ValueError(f"layer {layer.prefix}: the prenorm block is a norm and a mixer, and optionally a second norm with a feed-forward")
         self.prefix = layer.prefix
+        self.residual_scale = float(residual_scale)
         self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)
         self.mixer = build_part("mixer", layer.mixer, hidden_size=hidden_size)
-        self.norm_post = build_part("norm", layer.norm_post, hidden_size=hidden_size)
-        self.ffn = build_part("ffn", layer.ffn, hidden_size=hidden_size)
+        self.norm_post = build_part("norm", layer.norm_post, hidden_size=hidden_size) if layer.norm_post is not None else None
+        self.ffn = build_part("ffn", layer.ffn, hidden_size=hidden_size) if layer.ffn is not None else None
 
     def children(self):
-        return (self.norm_in, self.mixer, self.norm_post, self.ffn)
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_post, self.ffn) if p is not None)
 
     def entry_norm(self):
         return self.norm_in
 
-    def _mixer(self, h, ctx, binding, residual):
-        sink = _sink(self.mixer, residual, self.norm_post)
-        return self.mixer.forward(h, ctx, binding, sink=sink) if sink is not None else self.mixer.forward(h, ctx, binding)
+    def _scaled(self, delta):
+        """A sub-block's output with the block's factor (what was added to the stream by the sub-block itself has it already)."""
+        if self.residual_scale == 1.0 or isinstance(delta, ScaledRows):
+            return delta
+        return ScaledDelta(delta, self.residual_scale)
+
+    def _mixer(self, h, ctx, binding, residual, following):
+        sink = _sink(self.mixer, residual, self.norm_post if self.ffn is not None else following, self.residual_scale)
+        out = self.mixer.forward(h, ctx, binding, sink=sink) if sink is not None else self.mixer.forward(h, ctx, binding)
+        return self._scaled(out)
 
     def _ffn(self, h, ctx, residual, following):
-        sink = _sink(self.ffn, residual, following)
-        return self.ffn.forward(h, ctx, sink=sink) if sink is not None else self.ffn.forward(h, ctx)
+        sink = _sink(self.ffn, residual, following, self.residual_scale)
+        return self._scaled(self.ffn.forward(h, ctx, sink=sink) if sink is not None else self.ffn.forward(h, ctx))
 
     def forward(self, residual, pending, ctx, binding: MixerBinding, following=None):
         t = ctx.timer
         if t is None:
             h = normed_for(self.norm_in, self.mixer, residual, pending, ctx)
-            delta = self._mixer(h, ctx, binding, residual)
+            delta = self._mixer(h, ctx, binding, residual, following)
+            if self.ffn is None:
+                return residual, delta
             h = normed_for(self.norm_post, self.ffn, residual, delta, ctx)
             return residual, self._ffn(h, ctx, residual, following)
         t.enter("norm"); h = normed_for(self.norm_in, self.mixer, residual, pending, ctx); t.mark("norm")
-        t.enter("mixer"); delta = self._mixer(h, ctx, binding, residual); t.mark("mixer")
+        t.enter("mixer"); delta = self._mixer(h, ctx, binding, residual, following); t.mark("mixer")
+        if self.ffn is None:
+            return residual, delta
         t.enter("norm"); h = normed_for(self.norm_post, self.ffn, residual, delta, ctx); t.mark("norm")
         t.enter("ffn"); out = self._ffn(h, ctx, residual, following); t.mark("ffn")
         return residual, out
@@ -116,7 +131,10 @@ class OutputNormBlock(Block):
             h = pending.rows
         else:
             if pending is not None:                       # a delta some other arrangement left: it belongs to the stream
-                residual += pending.sum(torch.float32) if hasattr(pending, "parts") else pending.float()
+                if isinstance(pending, ScaledDelta):
+                    residual += pending.tensor()
+                else:
+                    residual += pending.sum(torch.float32) if hasattr(pending, "parts") else pending.float()
             h = residual if ctx.act_dtype == torch.float32 else ops.cast_rows(residual, ctx.act_dtype)
         if t is not None:
             t.enter("mixer")

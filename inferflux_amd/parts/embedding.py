@@ -1,6 +1,6 @@
 """Token embedding and the output head.
 
-Embedding: x[t] = E[id[t]], no scaling, widened to the float32 stream
+Embedding: x[t] = E[id[t]] (times ``scale`` where a model has one), widened to the float32 stream
 (runtime/backends/cuda/native/cuda_kernels.cu:674-689).  Head: logits = h Wlm^T in float; the
 reference rounds logits to the activation type before widening them
 (transformer_forward.cu:2686-2699), which is not copied: logits are produced in float32.
@@ -22,9 +22,12 @@ from .plan import ParamSpec
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02, tensor: Optional[str] = None):
-        """``tensor``: the table's full name in the model file where that is not ``<name>.weight``."""
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02, tensor: Optional[str] = None,
+                 scale: float = 1.0):
+        """``tensor``: the table's full name in the model file where that is not ``<name>.weight``; ``scale``: a factor
+        on every row."""
         self.name, self.vocab_size, self.hidden_size, self.init_std = name, int(vocab_size), int(hidden_size), init_std
+        self.scale = float(scale)
         self.tensor = tensor or f"{name}.weight"
         self.table: Optional[torch.Tensor] = None
 
@@ -43,8 +46,8 @@ class TokenEmbedding(Part):
         params = norm.rms_params() if norm is not None else None
         if (params is not None and 0 < ctx.n_tokens <= 16 and ctx.act_dtype == torch.bfloat16
                 and params[0].dtype == torch.bfloat16):
-            return ops.embedding_scaled(ctx.token_ids, self.table, params[0], params[1])
-        return ops.embedding(ctx.token_ids, self.table)
+            return ops.embedding_scaled(ctx.token_ids, self.table, params[0], params[1], self.scale)
+        return ops.embedding(ctx.token_ids, self.table, self.scale)
 
 
 @register_part("head", "linear_head")

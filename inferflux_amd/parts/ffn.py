@@ -1,4 +1,5 @@
-"""SwiGLU feed-forward: down( silu(gate(x)) * up(x) ), no biases.
+"""Gated feed-forward: down( act(gate(x)) * up(x) ), no biases; act is silu ("SwiGLU", the default) or the tanh form
+of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
 
 g = h Wg^T, u = h Wu^T, a = g / (1 + exp(-g)) * u in float, delta = a Wd^T
 (runtime/backends/cuda/native/transformer_forward.cu:2383-2419, 2487-2494, 2528-2547;
@@ -10,7 +11,7 @@ any output element.
 """
 from __future__ import annotations
 
-from typing import Dict, Mapping
+from typing import Dict, Mapping, Optional
 
 import torch
 
@@ -26,31 +27,43 @@ def concat_weights(parts):
     return torch.cat(list(parts), dim=0).contiguous()
 
 
+ACTIVATIONS = {"silu": ops.ACT_SILU, "gelu_tanh": ops.ACT_GELU_TANH}
+
+
+@register_part("ffn", "gated_ffn")
 @register_part("ffn", "swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
 
-    def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02):
+    def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02,
+                 activation: str = "silu", tensors: Optional[Mapping[str, str]] = None):
+        """``activation``: "silu" or "gelu_tanh".  ``tensors``: the full names of "gate", "up" and "down" in the model
+        file where they are not ``<name>.gate_proj.weight`` and so on."""
         self.name, self.hidden_size, self.intermediate_size = name, int(hidden_size), int(intermediate_size)
         self.init_std = init_std
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"{name}: activation '{activation}' unknown (one of {sorted(ACTIVATIONS)})")
+        self.activation, self.act = activation, ACTIVATIONS[activation]
+        self.names = {k: f"{name}.{k}_proj.weight" for k in ("gate", "up", "down")}
+        self.names.update(tensors or {})
         self.w_gate_up = None
         self.w_down = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         H, I, s = self.hidden_size, self.intermediate_size, ("normal", self.init_std)
         return {
-            f"{self.name}.gate_proj.weight": ParamSpec((I, H), s),
-            f"{self.name}.up_proj.weight": ParamSpec((I, H), s),
-            f"{self.name}.down_proj.weight": ParamSpec((H, I), s),
+            self.names["gate"]: ParamSpec((I, H), s),
+            self.names["up"]: ParamSpec((I, H), s),
+            self.names["down"]: ParamSpec((H, I), s),
         }
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        g, u = tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.w_gate_up = ops.prepare_linear(
             torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous())
-        self.w_down = ops.prepare_linear(tensors[f"{self.name}.down_proj.weight"])
+        self.w_down = ops.prepare_linear(tensors[self.names["down"]])
 
     adds_to_stream = True
 
@@ -58,9 +71,9 @@ class SwiGLU(FeedForward):
         return ops.takes_scaled_rows(n_rows, self.w_gate_up)
 
     def forward(self, h, ctx, sink=None):
-        a = ops.linear_swiglu(h, self.w_gate_up)
+        a = ops.linear_swiglu(h, self.w_gate_up, self.act)
         if ctx.timer is not None:
             ctx.timer.mark("ffn.gate_up")
         if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):
-            return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps)
+            return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps, sink.mult)
         return ops.linear(a, self.w_down, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself

@@ -84,8 +84,8 @@ class ModelPlan:
 class ParamSpec:
     """A tensor a part expects in the model file.
 
-    ``init`` is how the random-weights mode fills it: ("normal", std), ("ones",) or
-    ("zeros",).  ``integer`` tensors are kept as int32; floating tensors follow the
+    ``init`` is how the random-weights mode fills it: ("normal", std), ("ones",), ("zeros",),
+    ("uniform", lo, hi) or ("log_uniform", lo, hi) (the logarithm of a uniform number).  ``integer`` tensors are kept as int32; floating tensors follow the
     engine's dtype rule (see weights.loader).
     """
     shape: Tuple[int, ...]
@@ -100,12 +100,14 @@ class CacheSpec:
     ``v_head_dim`` (None: as wide as the keys).
 
     ``window`` is None when every past token stays readable, or the number of most recent
-    positions (the current one included) that the mixer reads; older pages are given back.
+    positions (the current one included) that the mixer reads; older pages are given back, except
+    those that hold any of the first ``keep_first`` positions, which a windowed mixer may go on reading.
     """
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    keep_first: int = 0
 
     @property
     def k_dim(self) -> int:
@@ -122,6 +124,7 @@ class CacheSpec:
 @dataclasses.dataclass(frozen=True)
 class StateSpec:
     """Fixed-size per-request state of a mixer: one tensor of ``shape`` per live request,
-    zero when the request starts."""
+    zero when the request starts.  A mixer that keeps several things (a recurrence's state and the last inputs of
+    a short convolution) lays them end to end in the one tensor."""
     shape: Tuple[int, ...]
     dtype: str = "float32"

@@ -12,9 +12,16 @@ cuda_kernels.cu:71-117): pair p joins elements p and p + d/2, f_p = 1 / theta^(2
 (x_p, x_{p+d/2}) <- (x_p cos a - x_{p+d/2} sin a, x_p sin a + x_{p+d/2} cos a).  The reference
 evaluates powf per element; here the d/2 frequencies are computed once in double precision
 and rounded to float.
+
+Frequencies scaled for contexts longer than the model was trained on ("YaRN", ``scaling`` = factor, original, fast,
+slow): with dim(t) = dims ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)),
+dims - 1) and ramp_p = clamp((p - lo) / max(hi - lo, 0.001), 0, 1), pair p turns with f_p / factor * ramp_p +
+f_p (1 - ramp_p): the fast pairs keep their frequency, the slow ones are stretched by the factor, and cos and sin are
+both multiplied by 0.1 ln(factor) + 1.
 """
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -50,7 +57,9 @@ class RotaryPosition(PositionEncoding):
 
     STYLES = {"split_half": ops.ROPE_SPLIT_HALF, "consecutive": ops.ROPE_CONSECUTIVE}
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, style: str = "split_half"):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, style: str = "split_half",
+                 scaling: Optional[dict] = None):
+        """``scaling``: None, or {"factor", "original", "fast", "slow"} (see the module's text)."""
         self.head_dim = int(head_dim)
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
         self.theta = float(theta)
@@ -59,19 +68,41 @@ class RotaryPosition(PositionEncoding):
         if self.rotary_dim % 2 or not (0 < self.rotary_dim <= self.head_dim):
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
         self.style = style
+        self.scaling = None
+        self.magnitude = 1.0
+        if scaling:
+            missing = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
+            if missing:
+                raise ValueError(f"rotary scaling needs {missing}")
+            self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
+            if self.scaling["factor"] <= 0 or self.scaling["original"] <= 0 or self.scaling["fast"] <= 0 or self.scaling["slow"] <= 0:
+                raise ValueError(f"rotary scaling: factor, original, fast and slow must be positive, got {self.scaling}")
+            self.magnitude = 0.1 * math.log(self.scaling["factor"]) + 1.0
         self._inv_freq = {}
+
+    def frequencies(self) -> torch.Tensor:
+        """The pairs' frequencies in double precision."""
+        n = self.rotary_dim // 2
+        p = torch.arange(n, dtype=torch.float64)
+        f = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64), 2.0 * p / self.rotary_dim)
+        if self.scaling is None:
+            return f
+        sc, dims = self.scaling, self.rotary_dim
+        dim_of = lambda turns: dims * math.log(sc["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+        lo = max(math.floor(dim_of(sc["fast"])), 0)
+        hi = min(math.ceil(dim_of(sc["slow"])), dims - 1)
+        ramp = torch.clamp((p - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / sc["factor"] * ramp + f * (1.0 - ramp)
 
     def inv_freq(self, device) -> torch.Tensor:
         key = str(device)
         t = self._inv_freq.get(key)
         if t is None:
-            p = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
-            t = (1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64), 2.0 * p / self.rotary_dim))
-            t = t.to(torch.float32).to(device)
+            t = self.frequencies().to(torch.float32).to(device)
             self._inv_freq[key] = t
         return t
 
     def kernel_args(self, ctx):
-        cos, sin = ctx.derived(("rotary_table", self.theta, self.rotary_dim),
-                               lambda: ops.rope_table(ctx.positions, self.inv_freq(ctx.device)))
+        key = ("rotary_table", self.theta, self.rotary_dim, tuple(sorted(self.scaling.items())) if self.scaling else None)
+        cos, sin = ctx.derived(key, lambda: ops.rope_table(ctx.positions, self.inv_freq(ctx.device), self.magnitude))
         return self.STYLES[self.style], self.rotary_dim, cos, sin

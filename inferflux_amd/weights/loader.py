@@ -137,6 +137,12 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, dev
         t = torch.empty(spec.shape, dtype=torch.float32, device=device)
         t.normal_(0.0, float(spec.init[1]), generator=g)
         return t.to(dtype)
+    if kind in ("uniform", "log_uniform"):       # U(lo, hi), or its logarithm
+        g = torch.Generator(device=device)
+        g.manual_seed(tensor_seed(seed, name))
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device)
+        t.uniform_(float(spec.init[1]), float(spec.init[2]), generator=g)
+        return (t.log() if kind == "log_uniform" else t).to(dtype)
     raise ValueError(f"tensor '{name}': unknown init rule {spec.init!r}")
 
 

@@ -80,9 +80,11 @@ class PagePool:
 
 @dataclasses.dataclass(frozen=True)
 class GroupSpec:
-    """A set of schedule entries whose caches share pages.  ``window`` None keeps everything."""
+    """A set of schedule entries whose caches share pages.  ``window`` None keeps everything; a windowed group
+    still keeps the pages that hold any of the first ``keep_first`` positions."""
     window: Optional[int]
     entries: Tuple[int, ...]
+    keep_first: int = 0
 
 
 @dataclasses.dataclass
@@ -205,7 +207,8 @@ class CacheManager:
                 continue
             dead_blocks = min(first_needed // self.page_size, len(r.tables[g]))
             t = r.tables[g]
-            for b in range(dead_blocks - 1, -1, -1):  # released blocks form a prefix: stop at the first -1
+            kept = self._blocks_for(spec.keep_first)
+            for b in range(dead_blocks - 1, kept - 1, -1):  # released blocks form a run behind the kept ones: stop at the first -1
                 if t[b] < 0:
                     break
                 self.pools[g].release(t[b])
