@@ -56,7 +56,7 @@ class PreNormBlock(Block):
 
     def __init__(self, layer: LayerSpec, hidden_size: int, residual_scale: float = 1.0):
         if layer.norm_in is None or layer.extra or (layer.ffn is None) != (layer.norm_post is None):
-            raise ValueError(f"layer {layer.prefix}: the prenorm block is a norm and a mixer, and optionally a second norm with a feed-forward")
+            raise ValueError(f"layer {layer.prefix}: the prenorm block is a norm and a mixer, optionally a second norm with a feed-forward, no more and no less")
         self.prefix = layer.prefix
         self.residual_scale = float(residual_scale)
         self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)

@@ -79,10 +79,11 @@ def sink_softmax_attention(q, k, v, scale, size, keep_first, sink=True):
     T, H, _ = q.shape
     G = k.shape[1]
     out = np.zeros((T, H, v.shape[2]))
+    i, j = np.arange(T)[:, None], np.arange(T)[None, :]
+    mask = (j <= i) & ((i - j < size if size is not None else True) | (j < keep_first))      # ``visible`` for all pairs
     for h in range(H):
         g = h // (H // G)
         s = (q[:, h] @ k[:, g].T) * scale                     # [T, T]
-        mask = np.array([[visible(i, j, size, keep_first) for j in range(T)] for i in range(T)])
         s = np.where(mask, s, -np.inf)
         m = np.maximum(s.max(axis=1, keepdims=True), 0.0 if sink else -np.inf)
         e = np.exp(s - m)
@@ -175,3 +176,11 @@ def forward(config, W, tokens, return_layers=False):
         layers.append(x.copy())
     logits = rms_norm(x, W["final.norm"], eps) @ W["head"].T
     return (logits, np.stack(layers)) if return_layers else logits
+
+
+def greedy_generate(config, W, prompt, n_new):
+    """``n_new`` tokens, each the first maximum of the last position's logits of the whole sequence so far."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(np.argmax(forward(config, W, ids)[-1])))
+    return ids[len(prompt):]
