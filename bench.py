@@ -74,6 +74,27 @@ DESIGN_SIZES = {
     "medium-wide-latent": (_mumusun_shape(2048, 8, 16, 128, 64, 128, 1536, 512, 2048, 64, 6, 1408, 8, 4),
                            _dense_twin(2048, 8, 16, 128, 2, 8448, 2048)),
 }
+# Layer sizes for the comparison of the Podurax design (attention with kept first tokens, a sink, unit norms, value mixing
+# and an output gate; a selective state-space recurrence; gated gelu feed-forward) with the dense decoder at equal width,
+# depth, heads, window and feed-forward size.  ``pattern`` is the order of mixers ("a" attention, "m" the recurrence),
+# repeated to the depth: the sizes with one kind alone say what each mechanism costs.
+def _podurax_shape(width, layers, heads, kv_heads, dim, window, ff, inner, state, dt_rank, pattern, vocab=32000):
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5 * 8.0, "v_mix": True,
+           "rot": {"base": 1e6, "dims": dim // 2, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+           "mask": {"size": window, "keep_first": 4}}
+    ssm = {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": 4}
+    mix = {"a": ("attention", att), "m": ("mamba1", ssm)}
+    return {"architecture": "Podurax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "residual_mult": 0.5, "layers": [{"type": mix[pattern[i % len(pattern)]][0], "mixer": mix[pattern[i % len(pattern)]][1],
+                                              "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+
+
+PODURAX_SIZES = {
+    "small": (_podurax_shape(1024, 8, 8, 2, 128, 1024, 2816, 2048, 16, 64, "aama"), _dense_twin(1024, 8, 8, 128, 2, 2816, 1024)),
+    "medium": (_podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "aama"), _dense_twin(2048, 8, 16, 128, 2, 5632, 2048)),
+    "medium-attention": (_podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "a"), _dense_twin(2048, 8, 16, 128, 2, 5632, 2048)),
+    "medium-recurrent": (_podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "m"), _dense_twin(2048, 8, 16, 128, 2, 5632, 2048)),
+}
 CONTEXT = 4096
 PROMPT = 2048
 DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
@@ -97,12 +118,14 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
-    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", *WORKLOADS], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", "podurax", *WORKLOADS], default="decode",
                     help="decode: the headline measurement; prefill: only the 2,048-token prefill, --steps times "
                          "(for profiles); mixed3b / long14b: whole workloads through the scheduler; mumusun: prefill and "
                          "decode of the Mumusun design beside the dense decoder at equal size (--size, --only-design)")
-    ap.add_argument("--size", choices=["all", *DESIGN_SIZES], default="all", help="--workload mumusun: which of its sizes")
-    ap.add_argument("--only-design", choices=["both", "mumusun", "dense"], default="both", help="--workload mumusun: which of the two models")
+    ap.add_argument("--size", choices=["all", *dict.fromkeys([*DESIGN_SIZES, *PODURAX_SIZES])], default="all",
+                    help="--workload mumusun / podurax: which of its sizes")
+    ap.add_argument("--only-design", choices=["both", "mumusun", "podurax", "dense"], default="both",
+                    help="--workload mumusun / podurax: which of the two models")
     ap.add_argument("--no-decode-weight-copy", action="store_true",
                     help="decode from the weights' plain rows instead of the tiled copy")
     ap.add_argument("--ceilings", action=argparse.BooleanOptionalAction, default=True,
@@ -139,6 +162,8 @@ def main() -> int:
     ops.decode_weight_copy = not args.no_decode_weight_copy
     if args.workload in WORKLOADS:
         return run_workload(args, WORKLOADS[args.workload])
+    if args.workload == "podurax":
+        return run_design_compare(args, PODURAX_SIZES, "podurax")
     if args.workload == "mumusun":
         return run_design_compare(args)
     shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B, "32b": SHAPE_32B,
@@ -435,8 +460,8 @@ def run_workload(args, w) -> int:
     return 0
 
 
-def run_design_compare(args) -> int:
-    """Prefill and decode throughput of the Mumusun design beside the dense decoder at equal size, through the step
+def run_design_compare(args, sizes=None, name="mumusun") -> int:
+    """Prefill and decode throughput of a design (``name``, its sizes in ``sizes``) beside the dense decoder at equal size, through the step
     function (no scheduler, no sampling): a prompt of --prompt-len tokens whole, and decode steps of 1, 8 and 64
     requests that each hold --context tokens.  One JSON line with every number."""
     import torch
@@ -449,10 +474,11 @@ def run_design_compare(args) -> int:
     dev = torch.device("cuda", 0)
     context = min(args.context, 1536)
     results = {}
-    for size, shapes in DESIGN_SIZES.items():
+    sizes = DESIGN_SIZES if sizes is None else sizes
+    for size, shapes in sizes.items():
         if args.size not in ("all", size):
             continue
-        for design, shape in zip(("mumusun", "dense"), shapes):
+        for design, shape in zip((name, "dense"), shapes):
             if args.only_design not in ("both", design):
                 continue
             cfg = config_from_dict(shape)
@@ -499,11 +525,12 @@ def run_design_compare(args) -> int:
             print(note, file=sys.stderr, flush=True)
             del runner, model
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prefill and decode tokens/s of the Mumusun design beside the dense decoder at equal size "
-                                f"({args.dtype}, random weights, {len(DESIGN_SIZES['small'][0]['layers'])} layers each)",
-                      "dtype": args.dtype, "data": "synthetic", "sizes": {k: {"mumusun": v[0]["layers"][0], "dense": {
+    first_of_each = lambda layers: list({L["type"]: L for L in layers}.values())      # one layer of every kind the size has
+    print(json.dumps({"metric": f"prefill and decode tokens/s of the {name.capitalize()} design beside the dense decoder at equal size "
+                                f"({args.dtype}, random weights, {len(sizes['small'][0]['layers'])} layers each)",
+                      "dtype": args.dtype, "data": "synthetic", "sizes": {k: {name: first_of_each(v[0]["layers"]), "dense": {
                           kk: v[1][kk] for kk in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size", "sliding_window")}}
-                          for k, v in DESIGN_SIZES.items() if args.size in ("all", k)},
+                          for k, v in sizes.items() if args.size in ("all", k)},
                       "results": results}), flush=True)
     return 0
 

@@ -68,12 +68,13 @@ struct RowBlock {
 
 template <bool STREAM>
 __device__ __forceinline__ void load_row_block(RowBlock& b, const RowArgs& a, int pages, int page_base, int kvh, int j0,
-                                               int ka, int kb, int col, int g4) {
+                                               int ka, int kb, int col, int g4, int ke = 0) {
+  // keys [ka, kb) are visible, and keys below ke (the kept first keys, where the walk passes them)
   const int P = a.P;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int k0 = j0 + 16 * t;  // 16 keys k0..k0+15, all in one page
-    bool live = k0 < kb && k0 + 16 > ka;
+    bool live = k0 < kb && (k0 + 16 > ka || k0 < ke);
     const int page = live ? __builtin_amdgcn_readlane(pages, k0 / P - page_base) : -1;
     live = live && page >= 0;
     b.live[t] = live;
@@ -90,7 +91,7 @@ __device__ __forceinline__ void load_row_block(RowBlock& b, const RowArgs& a, in
 }
 
 __device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& a, const bf16x8* qop, floatx4* o, float& m,
-                                              float& l, int j0, int ka, int kb, int g4) {
+                                              float& l, int j0, int ka, int kb, int g4, int ke = 0) {
   floatx4 s[2];
   float mb = -INFINITY;
 #pragma unroll
@@ -101,7 +102,7 @@ __device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& 
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int key = j0 + 16 * t + 4 * g4 + r;
-      const bool vis = b.live[t] && key >= ka && key < kb;
+      const bool vis = b.live[t] && (key >= ka || key < ke) && key < kb;
       s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
       mb = fmaxf(mb, s[t][r]);
     }
@@ -145,6 +146,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
+  // ... and of the kept first keys [0, keep) those of this split: [split * chunk, ke).  Where there are any the walk
+  // starts at the split's first key and passes whatever lies between them and the window without loading it.
+  const int keep = lo > 0 ? min(a.keep_first, lo) : 0;
+  const int ke = split * a.chunk < keep ? min(keep, min(pos + 1, (split + 1) * a.chunk)) : 0;
+  const int walk0 = ke > 0 ? split * a.chunk : ka;
   const int ratio = a.nH / a.nKV;
   const int* table = early ? early_table : a.block_table + (size_t)a.row_req[row] * a.max_blocks;
 
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     const bool head_ok = qt + col < ratio;
     float* po = a.part_o + (((size_t)ri * a.nH + head) * a.max_splits + split) * D;
     float* pml = a.part_ml + (((size_t)ri * a.nH + head) * a.max_splits + split) * 2;
-    if (ka >= kb) {  // nothing of this split is visible: the merge skips it
+    if (ka >= kb && ke == 0) {  // nothing of this split is visible: the merge skips it
       if (head_ok && g4 == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
       continue;
     }
@@ -169,7 +175,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     float m = -INFINITY, l = 0.f;
 
     RowBlock b0, b1;
-    int j0 = (ka / 32) * 32;
+    int j0 = (walk0 / 32) * 32;
     int page_base = early_base, pages = early_pages;
     bool have_pages = early;
     // the table entries of the block of 32 keys from j: in ``pages`` already, or read now (64 entries from j's)
@@ -180,20 +186,20 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
       pages = page_base + lane < a.max_blocks ? table[page_base + lane] : -1;
     };
     table_for(j0);
-    load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0, ka, kb, col, g4);
+    load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0, ka, kb, col, g4, ke);
     for (; j0 < kb; j0 += 64) {
       const bool more1 = j0 + 32 < kb, more2 = j0 + 64 < kb;
       if (more1) {
         table_for(j0 + 32);
-        load_row_block<STREAM>(b1, a, pages, page_base, kvh, j0 + 32, ka, kb, col, g4);
+        load_row_block<STREAM>(b1, a, pages, page_base, kvh, j0 + 32, ka, kb, col, g4, ke);
       }
-      use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4);
+      use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4, ke);
       if (more1) {
         if (more2) {
           table_for(j0 + 64);
-          load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0 + 64, ka, kb, col, g4);
+          load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0 + 64, ka, kb, col, g4, ke);
         }
-        use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4);
+        use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4, ke);
       }
     }
     l = col_sum(l);
@@ -230,10 +236,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  // this wave's keys: the visible ones from the first visible run of 32 on, in W equal shares of whole runs
+  // this wave's keys: the visible ones from the first visible run of 32 on, in W equal shares of whole runs.  With
+  // kept first keys [0, keep) before the window the runs are numbered as if the window's first run followed the last
+  // kept run: walk place v is key v below kr and key v + gap from there on.
   const int first = lo / 32 * 32;
-  const int chunk = ((pos + 1 - first + W - 1) / W + 31) / 32 * 32;
-  const int ka = max(lo, first + wid * chunk), kb = min(pos + 1, first + (wid + 1) * chunk);
+  const int keep = lo > 0 ? min(a.keep_first, lo) : 0;
+  const int keep_runs = (keep + 31) / 32 * 32;
+  const int base = keep > 0 ? 0 : first;
+  const int gap = (keep > 0 && keep_runs < first) ? first - keep_runs : 0, kr = gap > 0 ? keep_runs : 0;
+  const int vend = pos + 1 - gap;
+  const int chunk = ((vend - base + W - 1) / W + 31) / 32 * 32;
+  const int va = base + wid * chunk, vb = min(vend, base + (wid + 1) * chunk);     // this wave's places [va, vb), whole runs
+  const int ka = lo, kb = pos + 1, ke = keep;                                      // what is visible at all
+  auto key_at = [&](int v) { return v < kr ? v : v + gap; };
   const int ratio = a.nH / a.nKV;
   const int nc_max = min(16, ratio);
   const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
@@ -249,7 +264,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
-    if (ka < kb) {
+    if (va < vb) {
       bf16x8 qop[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -257,7 +272,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         qop[ks] = (head_ok && c < D) ? *(const bf16x8*)(a.q + ((size_t)row * a.nH + head) * D + c) : zero8();
       }
       RowBlock b0, b1;
-      int j0 = (ka / 32) * 32;
+      int j0 = va;
       int page_base = 0, pages = -1;
       bool have_pages = false;
       auto table_for = [&](int j) {
@@ -266,21 +281,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         page_base = j / a.P;
         pages = page_base + lane < a.max_blocks ? table[page_base + lane] : -1;
       };
-      table_for(j0);
-      load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0, ka, kb, col, g4);
-      for (; j0 < kb; j0 += 64) {
-        const bool more1 = j0 + 32 < kb, more2 = j0 + 64 < kb;
+      table_for(key_at(j0));
+      load_row_block<STREAM>(b0, a, pages, page_base, kvh, key_at(j0), ka, kb, col, g4, ke);
+      for (; j0 < vb; j0 += 64) {
+        const bool more1 = j0 + 32 < vb, more2 = j0 + 64 < vb;
         if (more1) {
-          table_for(j0 + 32);
-          load_row_block<STREAM>(b1, a, pages, page_base, kvh, j0 + 32, ka, kb, col, g4);
+          table_for(key_at(j0 + 32));
+          load_row_block<STREAM>(b1, a, pages, page_base, kvh, key_at(j0 + 32), ka, kb, col, g4, ke);
         }
-        use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4);
+        use_row_block(b0, a, qop, o, m, l, key_at(j0), ka, kb, g4, ke);
         if (more1) {
           if (more2) {
-            table_for(j0 + 64);
-            load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0 + 64, ka, kb, col, g4);
+            table_for(key_at(j0 + 64));
+            load_row_block<STREAM>(b0, a, pages, page_base, kvh, key_at(j0 + 64), ka, kb, col, g4, ke);
           }
-          use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4);
+          use_row_block(b1, a, qop, o, m, l, key_at(j0 + 32), ka, kb, g4, ke);
         }
       }
       l = col_sum(l);
@@ -309,7 +324,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] = fmaf(wgt, v[r], acc[r]);
       }
-      const float inv = L > 0.f ? 1.f / L : 0.f;
+      const float inv = finish_factor(M, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + kvh * ratio + qt + c);
       bf16x4 w4;
 #pragma unroll
       for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(acc[r] * inv);
@@ -327,7 +342,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
                              const int* row_req, const int* positions, const int* block_table, int max_blocks,
                              int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
                              int max_splits, float scale, float* part_o, float* part_ml, int waves, int req_is_row,
-                             void* stream) {
+                             int keep_first, int has_sink, float sink_score, const float* gate, void* stream) {
   IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
@@ -336,7 +351,8 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f, 0, waves, req_is_row};
+            scale * 1.4426950408889634f, 0, waves, req_is_row, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate};
+  IFX_REQUIRE(keep_first >= 0, "attn_rows: keep_first %d", keep_first);
   hipStream_t s = (hipStream_t)stream;
   const bool streaming = n_rows >= ROW_STREAM_MIN_ROWS && page_size == 16;
   if (waves > 0) {
@@ -399,6 +415,11 @@ struct TileArgs {
   // the i-th workgroup that XCD x is given.  The caller orders the items so that the workgroups that come to
   // share a compute unit have about the same number of key tiles between them on every unit.
   const int* order;
+  // Optional, off when zero (see RowArgs): the first keys a windowed row also sees, the sink, the gate [T, nH].
+  int keep_first = 0;
+  int has_sink = 0;
+  float sink_l2 = 0.f;
+  const float* gate = nullptr;
 };
 
 constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
@@ -535,7 +556,7 @@ struct QueryTile {
 
 template <bool MASKED>
 __device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, QueryTile* q, float c_log2e, int j0, int col,
-                                          int g4) {
+                                          int g4, int keep = 0) {
   floatx4 s[QT][4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -561,7 +582,7 @@ __device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, 
       for (int r = 0; r < 4; ++r) {
         if (MASKED) {
           const int key = j0 + 16 * t + 4 * g4 + r;
-          const bool vis = q[qt].ok && key <= q[qt].pos && key >= q[qt].lo;
+          const bool vis = q[qt].ok && key <= q[qt].pos && (key >= q[qt].lo || key < keep);
           s[qt][t][r] = vis ? s[qt][t][r] : -INFINITY;
         }
         mb = fmaxf(mb, s[qt][t][r]);
@@ -671,25 +692,38 @@ void attn_tiles_kernel(TileArgs a) {
   const int wave_hi = min(row_last, wave_first + 16 * QT - 1);
   const int wave_lo = a.window > 0 ? max(0, wave_first - a.window + 1) : 0;
 
+  // The walk: key tiles from the window's first to the last row's, and before them, where the rows keep their
+  // request's first keys [0, keep) and those end before the window's first tile, the tiles that hold them (of this
+  // split).  Tile n of the walk starts at key tile_at(n).
+  const int w0 = (lo_wg / TK) * TK;
+  const int keep = a.keep_first;        // (a row sees key j <= its position if j is in its window or below keep)
+  const int k0 = a.max_splits > 1 ? split * a.chunk : 0;                            // (a multiple of TK)
+  const int k1 = min(keep, pos_last + 1);                                           // kept keys of this split: [k0, k1)
+  const int n_kept = (k1 > k0 && (k1 + TK - 1) / TK * TK <= w0) ? (k1 - k0 + TK - 1) / TK : 0;
+  const int w_from = (k1 > k0 && n_kept == 0) ? k0 : w0;       // kept keys that reach the window's first tile: one walk from theirs
+  const int n_win = pos_last >= w_from ? (pos_last - w_from) / TK + 1 : 0;
+  const int n_walk = n_kept + n_win;
+  auto tile_at = [&](int n) { return n < n_kept ? k0 + n * TK : w_from + (n - n_kept) * TK; };
+
   TileRegs regs;
-  int j0 = (lo_wg / TK) * TK;
-  TilePages pg = tile_pages(a, table, j0, pos_last);
-  fetch_tile(regs, a, pg, kvh, j0, tid);
-  pg = tile_pages(a, table, j0 + TK, pos_last);
-  for (; j0 <= pos_last; j0 += TK) {
+  TilePages pg = tile_pages(a, table, tile_at(0), pos_last);
+  if (n_walk > 0) fetch_tile(regs, a, pg, kvh, tile_at(0), tid);
+  pg = tile_pages(a, table, tile_at(1), pos_last);
+  for (int n = 0; n < n_walk; ++n) {
+    const int j0 = tile_at(n);
     __syncthreads();  // everyone is done with the previous tile
     stage_tile(regs, k_s, v_s, tid);
     __syncthreads();
-    if (j0 + TK <= pos_last) {  // the next tile's data and the one after's pages: in flight during the arithmetic
-      fetch_tile(regs, a, pg, kvh, j0 + TK, tid);
-      pg = tile_pages(a, table, j0 + 2 * TK, pos_last);
+    if (n + 1 < n_walk) {  // the next tile's data and the one after's pages: in flight during the arithmetic
+      fetch_tile(regs, a, pg, kvh, tile_at(n + 1), tid);
+      pg = tile_pages(a, table, tile_at(n + 2), pos_last);
     }
-    if (j0 > wave_hi || j0 + TK <= wave_lo) continue;   // uniform over the wave; barriers are at the loop's top
+    if (j0 > wave_hi || (j0 + TK <= wave_lo && j0 >= keep)) continue;   // uniform over the wave; barriers are at the loop's top
 
     // A tile every key of which every row of this wave sees needs no mask: the common case.
     const bool full = j0 + TK - 1 <= wave_first && (a.window <= 0 || j0 >= wave_hi - a.window + 1);
     if (full) tile_math<false>(k_s, v_s, q, a.scale_log2e, j0, col, g4);
-    else tile_math<true>(k_s, v_s, q, a.scale_log2e, j0, col, g4);
+    else tile_math<true>(k_s, v_s, q, a.scale_log2e, j0, col, g4, keep);
   }
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
@@ -703,7 +737,7 @@ void attn_tiles_kernel(TileArgs a) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = q[qt].o[dt];
     } else {
-      const float inv = l > 0.f ? 1.f / l : 0.f;
+      const float inv = finish_factor(q[qt].m * a.scale_log2e, l, a.has_sink, a.sink_l2, a.gate, row * a.nH + head);
       bf16_t* orow = a.out + (row * a.nH + head) * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -725,8 +759,10 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
                               const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
                               int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                               float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
-                              const int* positions, const int* order, int order_per_xcd, int n_xcd, void* stream) {
+                              const int* positions, const int* order, int order_per_xcd, int n_xcd, int keep_first,
+                              int has_sink, float sink_score, const float* gate, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
+  IFX_REQUIRE(keep_first >= 0, "attn_tiles: keep_first %d", keep_first);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
   IFX_REQUIRE(nH <= 65535, "attn_tiles: too many heads for one launch");
@@ -740,7 +776,8 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (n_tiles == 0) return 0;
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
-             n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order};
+             n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order, window > 0 ? keep_first : 0, has_sink,
+             sink_score * 1.4426950408889634f, gate};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
   IFX_REQUIRE(!order || (order_per_xcd > 0 && (long long)n_xcd * order_per_xcd >= items && order_per_xcd <= items),
@@ -753,7 +790,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (max_splits > 1) {
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-              scale * 1.4426950408889634f, 1};
+              scale * 1.4426950408889634f, 1, 0, 0, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate};
     hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, m);
   }
   IFX_LAUNCH_CHECK();

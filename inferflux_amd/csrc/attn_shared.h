@@ -82,7 +82,27 @@ struct RowArgs {
   int part_by_row;        // partial results lie at the batch row's number (the tile kernel's), not at its place in ``rows``
   int waves;              // the row kernel that takes a (row, kv head) whole: waves per workgroup
   int req_is_row;         // row_req[r] == r for every row (a step of single tokens): table lookups need not wait for it
+  // Optional, off when zero.  keep_first: a windowed row also sees its request's first so many keys.  has_sink: a key
+  // without value whose score (times log2 e: sink_l2) joins the softmax's denominator.  gate [T, nH]: a factor on
+  // every head's output.
+  int keep_first = 0;
+  int has_sink = 0;
+  float sink_l2 = 0.f;
+  const float* gate = nullptr;
 };
+
+// The sink joins a finished (maximum M, sum L, unnormalised output) once, where the output is written: returns the
+// factor on the output, 1 / (L + 2^(sink - M)) (times the head's gate), with care for a maximum below the sink's score.
+__device__ __forceinline__ float finish_factor(float M, float L, int has_sink, float sink_l2, const float* gate, size_t gate_at) {
+  float f = 1.f;
+  if (has_sink) {
+    const float Ms = fmaxf(M, sink_l2);
+    f = M == -INFINITY ? 0.f : exp2f(M - Ms);
+    L = L * f + exp2f(sink_l2 - Ms);
+  }
+  const float inv = L > 0.f ? f / L : 0.f;
+  return gate ? inv * gate[gate_at] : inv;
+}
 
 // out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s.
 // One workgroup per (row, head).  A wave takes a run of consecutive splits: lane s first weighs split s of the run,
@@ -108,7 +128,9 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int first = lo / a.chunk, last = pos / a.chunk;  // first and last split that hold a visible key
+  // first and last split that hold a visible key (with kept first keys the walk starts at split 0: the splits between
+  // them and the window saw nothing and say so)
+  const int first = (a.keep_first > 0 && lo > 0) ? 0 : lo / a.chunk, last = pos / a.chunk;
   // this wave's run of them: runs of MERGE_RUN, longer ones only for rows that MERGE_MAX_WAVES such runs do not cover.
   // How a row is cut depends on the row alone, not on how many waves the launch has (it has enough: merge_waves), so
   // a row's result is the same bits in every launch that holds it.
@@ -122,6 +144,7 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
 #pragma unroll
   for (int c = 0; c < C; ++c) acc[c] = 0.f;
   float L = 0.f, M = -INFINITY;
+  float M_all = -INFINITY;
   if (s0 <= s1) {
     // Lane s of a round holds split sb + s; runs of more than 64 splits take further rounds.  The first
     // round's maxima and sums are kept from the pass that finds the maximum (the usual case is one round).
@@ -192,6 +215,7 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
     if (wid > 0) return;
     float Mall = -INFINITY;
     for (int w = 0; w < nw; ++w) Mall = fmaxf(Mall, ml_w[w][0]);
+    M_all = Mall;
     L = 0.f;
 #pragma unroll
     for (int c = 0; c < C; ++c) acc[c] = 0.f;
@@ -204,7 +228,8 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
       for (int c = 0; c < C; ++c) acc[c] = fmaf(f, acc_w[w][lane + c * WAVE], acc[c]);
     }
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  else M_all = M;
+  const float inv = finish_factor(M_all, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + head);
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     const int e = lane + c * WAVE;

@@ -232,31 +232,30 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     table = ctx.block_table(cache.group)
     keep_first = int(keep_first or 0) if window else 0
     extras = keep_first > 0 or sink is not None or gate is not None
-    if extras:
-        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate)
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
         # values of another width than the keys, or heads wider than a wave's registers hold: one shared kv head (attention
         # through a latent) has a matrix-core kernel of its own, everything else (32-bit, odd sizes) the plain kernel
-        if ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
+        if not extras and ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
             chunk, splits = ops.wide_launch_shape(T, nH, ctx.kv_bound)
             return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits)
-        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
+        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate)
     n_kv = cache.k.shape[1]
     # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.
     tiled = ctx.h_q_len >= TILE_MIN
     qt, splits, chunk = 1, 1, 0
     if tiled.any():
         qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], ctx.h_kv_len[tiled], nH, lambda t: ops.attention_tile_rows(d, t),
-                                          tall_direct=d == ops.DIRECT_TILE_HEAD_DIM)
+                                          tall_direct=d == ops.DIRECT_TILE_HEAD_DIM and not extras)
     tile_rows = ops.attention_tile_rows(d, qt)
     w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window, d),
                     lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window, ops.row_waves_fit(nH, n_kv, d, ops.ROW_MAX_WAVES)))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
+    more = dict(keep_first=keep_first, sink=sink, gate=gate) if extras else {}
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
                             table, window, scale, qt, w["tile_chunk"], w["tile_splits"], w["tile_row_list"], ctx.row_req,
-                            ctx.positions, w["tile_order"])
+                            ctx.positions, w["tile_order"], **more)
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
-                           window, scale, w["chunk"], w["max_splits"], w["waves"], ctx.n_tokens == ctx.n_requests)
+                           window, scale, w["chunk"], w["max_splits"], w["waves"], ctx.n_tokens == ctx.n_requests, **more)
     return out

@@ -63,13 +63,16 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
             yield _tile_module(d, qt)[:2]
+    if DIRECT_TILE_HEAD_DIM is not None:      # (tall tiles with kept first keys, a sink or a gate at that head size)
+        yield _tile_module(DIRECT_TILE_HEAD_DIM, 2, direct=False)[:2]
     for dk, dv in WIDE_DIMS_PREBUILT:
         yield ("attn_wide", (("K_DIM", dk), ("V_DIM", dv)))
 
 
-def _tile_module(head_dim: int, qt: int):
-    """(module, variant, entry point, the function that says its tile rows) of the tile kernel for a tiling."""
-    if qt == 2 and head_dim == DIRECT_TILE_HEAD_DIM:
+def _tile_module(head_dim: int, qt: int, direct: bool = True):
+    """(module, variant, entry point, the function that says its tile rows) of the tile kernel for a tiling.  ``direct``
+    False: not the kernel that loads straight into LDS (it has no kept first keys, sink or gate)."""
+    if qt == 2 and head_dim == DIRECT_TILE_HEAD_DIM and direct:
         return "attn_prefill", (("HEAD_DIM", head_dim),), "ifx_attn_prefill", "ifx_attn_prefill_tile_rows"
     return "attn_mfma", (("HEAD_DIM", head_dim), ("TILE_QT", qt)), "ifx_attn_tiles", "ifx_attn_tile_rows"
 
@@ -1174,7 +1177,7 @@ def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) 
             and page_size >= 16 and page_size & (page_size - 1) == 0)
 
 
-def _attn_common(q, k_cache, v_cache, qt=1):
+def _attn_common(q, k_cache, v_cache, qt=1, direct=True):
     _check(q, "q", (None, None, None), torch.bfloat16)
     T, nH, d = q.shape
     _check(k_cache, "k_cache", (None, None, None, d), torch.bfloat16)
@@ -1183,8 +1186,16 @@ def _attn_common(q, k_cache, v_cache, qt=1):
     if not mfma_attention_supported(q.dtype, d, page_size):
         raise KernelError(f"matrix-core attention needs bfloat16, head_dim a multiple of 16 up to {MFMA_MAX_HEAD_DIM} and "
                           f"page_size a power of two from 16; got head_dim {d}, page_size {page_size}")
-    name, variant, _, _ = _tile_module(d, qt)
+    name, variant, _, _ = _tile_module(d, qt, direct)
     return T, nH, d, nKV, page_size, load_module(name, variant)
+
+
+def _attn_extras(T, nH, keep_first, sink, gate):
+    """The four optional arguments of the matrix-core attention kernels: kept first keys, whether there is a sink, its
+    score, the gate's pointer."""
+    if gate is not None:
+        _check(gate, "gate", (T, nH), torch.float32)
+    return int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate)
 
 
 ROW_MAX_WAVES = 8
@@ -1201,8 +1212,10 @@ def row_waves_fit(n_heads: int, n_kv_heads: int, head_dim: int, waves: int) -> i
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                    rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
                    block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
-                   waves: int = 0, req_is_row: bool = False) -> None:
-    """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].
+                   waves: int = 0, req_is_row: bool = False, keep_first: int = 0, sink: Optional[float] = None,
+                   gate: Optional[torch.Tensor] = None) -> None:
+    """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].  ``keep_first``,
+    ``sink``, ``gate``: as for ``attention_plain``.
 
     ``waves`` 0: split s of a row covers key positions [s*chunk, (s+1)*chunk), one wave each, and a second launch
     merges a row's splits; ``max_splits`` * chunk must reach past the largest position among the rows.
@@ -1228,10 +1241,11 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
     if req_is_row and block_table.shape[0] < T:
         raise KernelError("attention_rows: req_is_row needs a block-table row for every row of the step")
-    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, P),
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, I, I, F, P, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
-          int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, 1 if req_is_row else 0, _stream())
+          int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, 1 if req_is_row else 0,
+          *_attn_extras(T, nH, keep_first, sink, gate), _stream())
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
@@ -1245,7 +1259,8 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float,
                     qt: int = 1, chunk: int = 0, max_splits: int = 1, rows: Optional[torch.Tensor] = None,
                     row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
-                    order: Optional[torch.Tensor] = None) -> None:
+                    order: Optional[torch.Tensor] = None, keep_first: int = 0, sink: Optional[float] = None,
+                    gate: Optional[torch.Tensor] = None) -> None:
     """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
     request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d].
 
@@ -1256,8 +1271,9 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
     ``order`` (int32 [8 * n], from ``attention.tile_order``) says which work item each workgroup of the launch
     takes; every item must appear exactly once (-1: a workgroup without work).  The result does not depend on it."""
-    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
-    _, _, entry, rows_fn = _tile_module(d, qt)
+    extras = bool(keep_first) or sink is not None or gate is not None      # (the kernel that loads straight into LDS has none of them)
+    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt, not extras)
+    _, _, entry, rows_fn = _tile_module(d, qt, not extras)
     if mod.fn(rows_fn, ())() != attention_tile_rows(d, qt):
         raise KernelError("attention_tiles: the compiled module's tile rows differ from attention_tile_rows()")
     _check(out, "out", (T, nH * d), torch.bfloat16)
@@ -1287,11 +1303,15 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if order.shape[0] % N_XCD:
             raise KernelError(f"attention_tiles: the order has a place for each of {N_XCD} XCDs' workgroups")
         per_xcd = order.shape[0] // N_XCD
-    _call(mod, entry, (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, I, P),
-          q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
-          n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
-          block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),
-          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, N_XCD, _stream())
+    args = (q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
+            n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
+            block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),
+            _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, N_XCD)
+    types = (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, I)
+    if entry == "ifx_attn_tiles":
+        _call(mod, entry, types + (I, I, F, P, P), *args, *_attn_extras(T, nH, keep_first, sink, gate), _stream())
+    else:
+        _call(mod, entry, types + (P,), *args, _stream())
 
 
 # ----------------------------------------------------------------------------------------
