@@ -122,27 +122,71 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log
 // LANES lanes share a channel, each with NPT of its states (state n belongs to lane n / NPT); a token's sum over the
 // states is added across them in a fixed order.  TOK tokens' inputs are asked for together, so that the recurrence,
 // which is a chain from token to token, waits for memory once per TOK tokens.
+//
+// MODE 0: a workgroup row (blockIdx.y) is a request; its rows of the step are walked in order from the state in its
+// slot, which receives the new state.  This is the whole scan for steps of few rows per request, and the only one in
+// 32-bit, where a token's arithmetic must not depend on how its request was cut into steps.
+// MODES 1-3 cut long portions into chunks that run side by side (the recurrence is linear in S: the state after a
+// chunk is decay * (state before) + (state after the chunk from zero), decay = exp(A * sum of the chunk's dt)):
+//   1  a workgroup row is a chunk: from S = 0 over the chunk's rows; writes the final S and the sum of dt, no output
+//   2  a workgroup row is a request: walks its chunks, turns each chunk's entry into the state the chunk starts from,
+//      and leaves the request's new state in its slot
+//   3  a workgroup row is a chunk: from the state of pass 2 over the chunk's rows; writes the output
 constexpr int LANES = 4, TOK = 4;
 
-template <typename T, int NPT>
-__global__ __launch_bounds__(256) void scan_kernel(ScanArgs a) {
+struct ChunkArgs {
+  const int* chunk_req;    // [n_chunks] the request (place in the step) of each chunk
+  const int* chunk_t0;     // [n_chunks] its first row of the step
+  const int* chunk_len;    // [n_chunks]
+  const int* req_chunk0;   // [R + 1] a request's chunks are req_chunk0[r] .. req_chunk0[r + 1] - 1
+  float* chunk_state;      // [n_chunks, C, N]
+  float* chunk_dt;         // [n_chunks, C]
+};
+
+template <typename T, int NPT, int MODE>
+__global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  const int c = idx / LANES, lg = idx % LANES, r = blockIdx.y;
+  const int c = idx / LANES, lg = idx % LANES;
   if (c >= a.C) return;          // (C * LANES is a multiple of LANES: the lanes of a channel leave together)
   const int N = a.N, n0 = lg * NPT;
-  const int t0 = a.q_start[r], n_tok = a.q_len[r];
-  float* S_mem = a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + (size_t)c * N + n0;
-  float S[NPT], An[NPT];
+  float An[NPT];
 #pragma unroll
-  for (int k = 0; k < NPT; ++k) {
-    const bool ok = n0 + k < N;
-    S[k] = ok ? S_mem[k] : 0.f;
-    An[k] = ok ? a.A[(size_t)c * N + n0 + k] : 0.f;
+  for (int k = 0; k < NPT; ++k) An[k] = n0 + k < N ? a.A[(size_t)c * N + n0 + k] : 0.f;
+  if (MODE == 2) {
+    const int r = blockIdx.y;
+    float* S_mem = a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + (size_t)c * N + n0;
+    float S[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) S[k] = n0 + k < N ? S_mem[k] : 0.f;
+    for (int q = ch.req_chunk0[r]; q < ch.req_chunk0[r + 1]; ++q) {
+      float* cs = ch.chunk_state + ((size_t)q * a.C + c) * N + n0;
+      const float sum_dt = ch.chunk_dt[(size_t)q * a.C + c];
+#pragma unroll
+      for (int k = 0; k < NPT; ++k)
+        if (n0 + k < N) {
+          const float local = cs[k];
+          cs[k] = S[k];
+          S[k] = fmaf(expf(sum_dt * An[k]), S[k], local);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NPT; ++k)
+      if (n0 + k < N) S_mem[k] = S[k];
+    return;
   }
+  const int item = blockIdx.y;
+  const int r = MODE == 0 ? item : ch.chunk_req[item];
+  const int t0 = MODE == 0 ? a.q_start[r] : ch.chunk_t0[item], n_tok = MODE == 0 ? a.q_len[r] : ch.chunk_len[item];
+  float* S_mem = MODE == 0 ? a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + (size_t)c * N + n0
+                           : ch.chunk_state + ((size_t)item * a.C + c) * N + n0;
+  float S[NPT];
+#pragma unroll
+  for (int k = 0; k < NPT; ++k) S[k] = (MODE != 1 && n0 + k < N) ? S_mem[k] : 0.f;
   const float dtb = load_dyn(a.dt_bias, a.w_dtype, c), Dc = load_dyn(a.D, a.w_dtype, c);
   const T* u = (const T*)a.u;
   const T* bc = (const T*)a.bc;
   const T* z = (const T*)a.z;
+  float sum_dt = 0.f;
   for (int i0 = 0; i0 < n_tok; i0 += TOK) {
     float uv[TOK], dtv[TOK], zv[TOK], Bv[TOK][NPT], Cv[TOK][NPT];
 #pragma unroll
@@ -151,18 +195,19 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a) {
       const size_t t = (size_t)t0 + i0 + (live ? q : 0);
       uv[q] = to_f(u[t * a.C + c]);
       dtv[q] = a.dt_raw[t * a.C + c];
-      zv[q] = to_f(z[t * a.ld_z + c]);
+      zv[q] = MODE == 1 ? 0.f : to_f(z[t * a.ld_z + c]);
 #pragma unroll
       for (int k = 0; k < NPT; ++k) {
         const int n = min(n0 + k, N - 1);
         Bv[q][k] = to_f(bc[t * a.ld_bc + n]);
-        Cv[q][k] = to_f(bc[t * a.ld_bc + N + n]);
+        Cv[q][k] = MODE == 1 ? 0.f : to_f(bc[t * a.ld_bc + N + n]);
       }
     }
 #pragma unroll
     for (int q = 0; q < TOK; ++q) {
       if (i0 + q >= n_tok) break;
       const float dt = softplus_f(dtv[q] + dtb), dtu = dt * uv[q];
+      sum_dt += dt;
       float y = 0.f;
 #pragma unroll
       for (int k = 0; k < NPT; ++k) {
@@ -171,24 +216,37 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a) {
           y = fmaf(S[k], Cv[q][k], y);
         }
       }
-      y += __shfl_xor(y, 1, WAVE);      // the channel's four lanes are neighbours
-      y += __shfl_xor(y, 2, WAVE);
-      if (lg == 0) {
-        y = fmaf(Dc, uv[q], y);
-        ((T*)a.out)[((size_t)t0 + i0 + q) * a.C + c] = from_f<T>(y * act_silu(zv[q]));
+      if (MODE != 1) {
+        y += __shfl_xor(y, 1, WAVE);      // the channel's four lanes are neighbours
+        y += __shfl_xor(y, 2, WAVE);
+        if (lg == 0) {
+          y = fmaf(Dc, uv[q], y);
+          ((T*)a.out)[((size_t)t0 + i0 + q) * a.C + c] = from_f<T>(y * act_silu(zv[q]));
+        }
       }
     }
   }
+  if (MODE == 3) return;
 #pragma unroll
   for (int k = 0; k < NPT; ++k)
     if (n0 + k < N) S_mem[k] = S[k];
+  if (MODE == 1 && lg == 0) ch.chunk_dt[(size_t)item * a.C + c] = sum_dt;
 }
 
 template <typename T>
-static int launch_scan(const ScanArgs& a, hipStream_t s) {
+static int launch_scan(const ScanArgs& a, const ChunkArgs& ch, int n_chunks, hipStream_t s) {
   const int npt = (a.N + LANES - 1) / LANES;
-  const dim3 grid((unsigned)(((size_t)a.C * LANES + 255) / 256), a.R);
-#define GO(NPT_) hipLaunchKernelGGL((scan_kernel<T, NPT_>), grid, dim3(256), 0, s, a)
+  const unsigned gx = (unsigned)(((size_t)a.C * LANES + 255) / 256);
+  const dim3 grid(gx, a.R), grid_chunks(gx, n_chunks > 0 ? n_chunks : 1);
+#define GO(NPT_)                                                                                  \
+  do {                                                                                            \
+    if (n_chunks <= 0) hipLaunchKernelGGL((scan_kernel<T, NPT_, 0>), grid, dim3(256), 0, s, a, ch); \
+    else {                                                                                        \
+      hipLaunchKernelGGL((scan_kernel<T, NPT_, 1>), grid_chunks, dim3(256), 0, s, a, ch);         \
+      hipLaunchKernelGGL((scan_kernel<T, NPT_, 2>), grid, dim3(256), 0, s, a, ch);                \
+      hipLaunchKernelGGL((scan_kernel<T, NPT_, 3>), grid_chunks, dim3(256), 0, s, a, ch);         \
+    }                                                                                             \
+  } while (0)
   if (npt <= 1) GO(1);
   else if (npt <= 2) GO(2);
   else if (npt <= 4) GO(4);
@@ -205,7 +263,12 @@ static int launch_scan(const ScanArgs& a, hipStream_t s) {
 extern "C" int ifx_selective_scan(const void* u, int dtype, const float* dt_raw, const void* dt_bias, const float* A,
                                   const void* bc, int ld_bc, const void* D, int w_dtype, const void* z, int ld_z,
                                   float* state, long long state_stride, long long state_offset, const int* q_start,
-                                  const int* q_len, const int* slots, void* out, int T, int R, int C, int N, void* stream) {
+                                  const int* q_len, const int* slots, void* out, int T, int R, int C, int N,
+                                  int n_chunks, const int* chunk_req, const int* chunk_t0, const int* chunk_len,
+                                  const int* req_chunk0, float* chunk_state, float* chunk_dt, void* stream) {
+  IFX_REQUIRE(n_chunks >= 0 && n_chunks <= 65535, "selective_scan: %d chunks", n_chunks);
+  IFX_REQUIRE(n_chunks == 0 || (chunk_req && chunk_t0 && chunk_len && req_chunk0 && chunk_state && chunk_dt),
+              "selective_scan: chunks need their lists and scratch");
   IFX_REQUIRE(T >= 0 && R >= 0 && C > 0 && N > 0, "selective_scan: bad sizes T=%d R=%d C=%d N=%d", T, R, C, N);
   IFX_REQUIRE(ld_bc >= 2 * N && ld_z >= C, "selective_scan: rows of %d for B and C of %d, of %d for a gate of %d", ld_bc, N, ld_z, C);
   IFX_REQUIRE(state_stride >= state_offset + (long long)C * N, "selective_scan: a state row of %lld floats for %lld + %d x %d", state_stride, state_offset, C, N);
@@ -213,7 +276,8 @@ extern "C" int ifx_selective_scan(const void* u, int dtype, const float* dt_raw,
   if (T == 0 || R == 0) return 0;
   ScanArgs a{u, dt_raw, dt_bias, A, bc, ld_bc, D, w_dtype, z, ld_z, state, (size_t)state_stride, (size_t)state_offset,
              q_start, q_len, slots, out, R, C, N};
-  if (dtype == DT_F32) return launch_scan<float>(a, (hipStream_t)stream);
-  if (dtype == DT_BF16) return launch_scan<bf16_t>(a, (hipStream_t)stream);
+  const ChunkArgs ch{chunk_req, chunk_t0, chunk_len, req_chunk0, chunk_state, chunk_dt};
+  if (dtype == DT_F32) return launch_scan<float>(a, ch, n_chunks, (hipStream_t)stream);
+  if (dtype == DT_BF16) return launch_scan<bf16_t>(a, ch, n_chunks, (hipStream_t)stream);
   IFX_FAIL("selective_scan: unknown dtype %d", dtype);
 }

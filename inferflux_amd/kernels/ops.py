@@ -1095,12 +1095,16 @@ def causal_conv_silu(x: torch.Tensor, channels: int, weight: torch.Tensor, bias:
 
 def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, bc: torch.Tensor,
                    D: torch.Tensor, z: torch.Tensor, state: torch.Tensor, state_offset: int, q_start: torch.Tensor,
-                   q_len: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+                   q_len: torch.Tensor, slots: torch.Tensor, chunks: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
     """The recurrence of a selective state-space mixer over each request's rows, then the gate:
     dt = softplus(dt_raw + dt_bias); S[c, n] <- exp(dt A[c, n]) S[c, n] + dt u[c] B[n]; y[c] = sum_n S[c, n] C[n] + D[c] u[c];
     out = y * silu(z).  ``u`` [T, C], ``dt_raw`` float32 [T, C], ``A`` float32 [C, N] (negative), ``bc`` [T, >= 2N] with B
     then C, ``z`` a view [T, C] of rows that may be wider (its row stride is taken), ``state`` float32 [slots, n] with a
-    request's S at ``state_offset`` of its row.  All of the recurrence is float.  Returns [T, C] in u's type."""
+    request's S at ``state_offset`` of its row.  All of the recurrence is float.  Returns [T, C] in u's type.
+
+    ``chunks`` (from ``scan_chunks``): the requests' rows cut into chunks that run side by side, each first from a zero
+    state, then from the state that the chunks before it leave (the recurrence is linear in S); the same function up to
+    the rounding of float sums taken in another order."""
     _check(u, "u", (None, None))
     T, C = u.shape
     _check(dt_raw, "dt_raw", (T, C), torch.float32)
@@ -1116,11 +1120,38 @@ def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
     for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
         _check(t, nm, (R,), torch.int32)
     out = torch.empty((T, C), dtype=u.dtype, device=u.device)
-    _call(load_module("ssm"), "ifx_selective_scan", (P, I, P, P, P, P, I, P, I, P, I, P, LL, LL, P, P, P, P, I, I, I, I, P),
+    n_chunks, lists = 0, (0, 0, 0, 0, 0, 0)
+    if chunks is not None:
+        n_chunks = chunks["req"].shape[0]
+        for nm in ("req", "t0", "len"):
+            _check(chunks[nm], f"chunks.{nm}", (n_chunks,), torch.int32)
+        _check(chunks["req_chunk0"], "chunks.req_chunk0", (R + 1,), torch.int32)
+        chunk_state = torch.empty((n_chunks, C, N), dtype=torch.float32, device=u.device)
+        chunk_dt = torch.empty((n_chunks, C), dtype=torch.float32, device=u.device)
+        lists = (chunks["req"].data_ptr(), chunks["t0"].data_ptr(), chunks["len"].data_ptr(), chunks["req_chunk0"].data_ptr(),
+                 chunk_state.data_ptr(), chunk_dt.data_ptr())
+    _call(load_module("ssm"), "ifx_selective_scan",
+          (P, I, P, P, P, P, I, P, I, P, I, P, LL, LL, P, P, P, P, I, I, I, I, I, P, P, P, P, P, P, P),
           u.data_ptr(), _dt(u), dt_raw.data_ptr(), dt_bias.data_ptr(), A.data_ptr(), bc.data_ptr(), bc.shape[1], D.data_ptr(),
           _dt(D), z.data_ptr(), z.stride(0) if T else C, state.data_ptr(), state.shape[1], int(state_offset), q_start.data_ptr(),
-          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, C, N, _stream())
+          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, C, N, n_chunks, *lists, _stream())
     return out
+
+
+def scan_chunks(q_start, q_len, chunk: int, device) -> Dict[str, torch.Tensor]:
+    """The lists ``selective_scan`` takes as ``chunks``: every request's rows (host arrays ``q_start`` / ``q_len`` of the
+    step) cut into chunks of up to ``chunk`` rows, in one upload."""
+    import numpy as np
+    req, t0, ln, first = [], [], [], [0]
+    for r, (s0, n) in enumerate(zip(q_start.tolist(), q_len.tolist())):
+        for at in range(0, n, chunk):
+            req.append(r); t0.append(s0 + at); ln.append(min(chunk, n - at))
+        first.append(len(req))
+    n = len(req)
+    pad = lambda v: v + [0] * (-len(v) % 4)
+    packed = torch.from_numpy(np.asarray(pad(req) + pad(t0) + pad(ln) + first, dtype=np.int32)).to(device)
+    w = n + -n % 4
+    return {"req": packed[:n], "t0": packed[w:w + n], "len": packed[2 * w:2 * w + n], "req_chunk0": packed[3 * w:3 * w + len(first)]}
 
 
 WIDE_MAX_K_DIM, WIDE_MAX_V_DIM = 1024, 512

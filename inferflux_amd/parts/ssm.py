@@ -35,6 +35,10 @@ from .base import Mixer, MixerBinding, register_part
 from .plan import ParamSpec, StateSpec
 
 
+SCAN_CHUNK = 64             # rows of a chunk of the scan where long portions are cut into chunks that run side by side
+SCAN_CHUNK_MIN_ROWS = 128   # ... which happens in steps that bring some request this many rows or more
+
+
 @register_part("mixer", "selective_ssm")
 class SelectiveSSM(Mixer):
     graph_safe = True          # every kernel reads the step's layout from the context's device arrays
@@ -100,8 +104,15 @@ class SelectiveSSM(Mixer):
         d = ops.linear(u, self.w_x_dt)                                  # [T, dt_rank]
         bc = ops.linear(u, self.w_x_bc)                                 # [T, 2 state]: B | C
         dt_raw = ops.linear(d, self.w_dt, out_dtype=torch.float32)      # [T, inner] float: the step sizes are never rounded
+        # A prompt's portion walked token by token leaves most of the chip idle (the recurrence of a channel is a chain):
+        # in bfloat16 long portions are cut into chunks that run side by side.  In 32-bit the walk stays in one piece, so
+        # that a token's sums do not depend on where its request was cut.  (Steps of single tokens, the ones that are
+        # captured and replayed, never take the chunks: a layout's launches stay the same.)
+        chunks = None
+        if u.dtype == torch.bfloat16 and ctx.n_tokens > ctx.n_requests and int(ctx.h_q_len.max()) >= SCAN_CHUNK_MIN_ROWS:
+            chunks = ctx.derived(("scan_chunks", SCAN_CHUNK), lambda: ops.scan_chunks(ctx.h_q_start, ctx.h_q_len, SCAN_CHUNK, ctx.device))
         y = ops.selective_scan(u, dt_raw, self.dt_b, self.A, bc, self.D, xz[:, C:], state, self.conv_floats,
-                               ctx.q_start, ctx.q_len, ctx.state_slots)
+                               ctx.q_start, ctx.q_len, ctx.state_slots, chunks)
         if t is not None:
             t.mark("mixer.scan")
         if sink is not None and ops.adds_into_stream(y.shape[0], self.w_o, sink.norm_weight):

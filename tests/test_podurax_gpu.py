@@ -331,6 +331,31 @@ def test_selective_scan_carries_its_state_from_step_to_step(dtype, C, N):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("C,N,chunk", [(96, 6, 64), (40, 17, 16), (256, 16, 64), (50, 5, 7), (24, 1, 200)])
+def test_selective_scan_in_chunks_side_by_side(dtype, C, N, chunk):
+    """Long portions cut into chunks that first run from zero and then from what the chunks before them leave: the same
+    outputs and the same final state as the walk in one piece, for requests of unequal length that start from a state."""
+    dt = DT[dtype]
+    lens = [300, 1, 70, 129]
+    T = sum(lens)
+    u, z, bc = rnd(70, T, C).to(dt), rnd(71, T, C).to(dt), rnd(72, T, 2 * N).to(dt)
+    dt_raw = rnd(73, T, C, scale=2.0).float()
+    dt_b, D = (rnd(74, C) - 2.0).to(dt), (rnd(75, C, scale=0.5) + 1.0).to(dt)
+    A = -torch.exp(torch.log(1.0 + 15.0 * torch.rand(C, N, generator=torch.Generator().manual_seed(76)))).float()
+    q_start, q_len, _ = _step_arrays(lens)
+    slots = torch.tensor([2, 0, 3, 1], dtype=torch.int32)
+    start = rnd(77, 4, C * N).float()
+    outs, states = [], []
+    for chunks in (None, ops.scan_chunks(q_start.numpy(), q_len.numpy(), chunk, DEV)):
+        state = start.clone().to(DEV)
+        outs.append(ops.selective_scan(u.to(DEV), dt_raw.to(DEV), dt_b.to(DEV), A.to(DEV), bc.to(DEV), D.to(DEV), z.to(DEV), state, 0,
+                                       q_start.to(DEV), q_len.to(DEV), slots.to(DEV), chunks).cpu())
+        states.append(state.cpu())
+    assert rel_err(outs[1], outs[0]) < (2e-5 if dtype == "float32" else 1e-2)
+    assert rel_err(states[1], states[0]) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("M", [1, 7, 16, 40, 100, 300])
 @pytest.mark.parametrize("K,ff", [(64, 96), (320, 320), (100, 50)])
 def test_gated_feed_forward_with_the_tanh_form_of_gelu(dtype, M, K, ff):
