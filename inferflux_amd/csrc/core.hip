@@ -580,6 +580,116 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
   }
 }
 
+// The same in 16-byte pieces for rows with the optional steps (unit norms, gate, value mixing, a rotation over part of
+// the head): bfloat16, split-half pairs, head size 16, 32, 64 or 128, rotated and unrotated parts both multiples of 16.
+// A head is d / 16 threads, each with two pieces of 8: in the rotated part piece j and its partner rot / 2 further, behind
+// it two neighbours.  The head's sum of squares is added across its threads by shuffles.  The other blocks append v as
+// above, dv wide, mixed and handed on where asked.
+__global__ __launch_bounds__(256) void rope_append_vec_x_kernel(RopeArgs a, int T, int n_qk_blocks) {
+  const int d = a.d, dv = a.dv, rot = a.rope_style != 0 ? a.rotary_dim : 0;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, v_width = a.nKV * dv, row_width = q_width + kv_width + v_width + a.gate_cols;
+  const bf16_t* qkv = (const bf16_t*)a.qkv;
+  const bf16_t* bias = (const bf16_t*)a.bias;
+  if ((int)blockIdx.x < n_qk_blocks) {
+    const int per_head = d / 16, heads = a.nH + (a.slots ? a.nKV : 0);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)T * heads * per_head) return;      // (whole heads leave together)
+    const int j = (int)(idx % per_head), head = (int)(idx / per_head % heads), t = (int)(idx / per_head / heads);
+    const bool rotate = 16 * j < rot;
+    const int first = rotate ? 8 * j : rot + 16 * (j - rot / 16), second = rotate ? first + rot / 2 : first + 8;
+    const bf16_t* row = qkv + (size_t)t * row_width + head * d;
+    const rope_bf16x8 x0 = *(const rope_bf16x8*)(row + first), x1 = *(const rope_bf16x8*)(row + second);
+    float f0[8], f1[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { f0[e] = (float)x0[e]; f1[e] = (float)x1[e]; }
+    if (bias) {
+      const rope_bf16x8 b0 = *(const rope_bf16x8*)(bias + head * d + first), b1 = *(const rope_bf16x8*)(bias + head * d + second);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { f0[e] += (float)b0[e]; f1[e] += (float)b1[e]; }
+    }
+    if (rotate) {
+      const float* cs = a.cs + (size_t)t * (rot / 2) + 8 * j;
+      const float* sn = a.sn + (size_t)t * (rot / 2) + 8 * j;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float u = f0[e], w = f1[e];
+        f0[e] = u * cs[e] - w * sn[e];
+        f1[e] = u * sn[e] + w * cs[e];
+      }
+    }
+    float inv = 1.f;
+    if (a.unit_norm) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f0[e] * f0[e] + f1[e] * f1[e];
+      for (int o = per_head / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);     // the head's threads are neighbours
+      inv = rsqrtf(ss / (float)d + a.norm_eps);
+    }
+    if (head < a.nH && a.gate_cols && j == 0) {
+      const int gc = q_width + kv_width + v_width + head;
+      float g = (float)qkv[(size_t)t * row_width + gc];
+      if (bias) g += (float)bias[gc];
+      a.gate_out[(size_t)t * a.nH + head] = 1.0f / (1.0f + expf(-g));
+    }
+    rope_bf16x8 y0, y1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { y0[e] = (__bf16)(f0[e] * inv); y1[e] = (__bf16)(f1[e] * inv); }
+    bf16_t* dst;
+    if (head < a.nH) {
+      dst = (bf16_t*)a.q_out + (size_t)t * q_width + head * d;
+    } else {
+      const int slot = a.slots[t];
+      if (slot < 0) return;
+      const int page = slot / a.page_size, off = slot % a.page_size;
+      dst = (bf16_t*)a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.page_size + off) * d;
+    }
+    *(rope_bf16x8*)(dst + first) = y0;
+    *(rope_bf16x8*)(dst + second) = y1;
+    return;
+  }
+  // v: (group of 8 tokens, kv head, dimension)
+  const size_t idx = (size_t)(blockIdx.x - n_qk_blocks) * 256 + threadIdx.x;
+  const int groups = (T + 7) / 8;
+  if (idx >= (size_t)groups * a.nKV * dv) return;
+  const int e = (int)(idx % dv), kh = (int)(idx / dv % a.nKV), t0 = (int)(idx / dv / a.nKV) * 8;
+  const int col = q_width + kv_width + kh * dv + e;
+  const float b = bias ? (float)bias[col] : 0.f;
+  const bf16_t* vf = (const bf16_t*)a.v_first;
+  bf16_t* vo = (bf16_t*)a.v_out;
+  int slot[8];
+  float x[8], m[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {   // all loads of the group are independent: they go out together
+    const bool live = t0 + k < T;
+    slot[k] = live && a.slots ? a.slots[t0 + k] : -1;
+    x[k] = live ? (float)qkv[(size_t)(t0 + k) * row_width + col] + b : 0.f;
+    m[k] = live && vf ? (float)vf[((size_t)(t0 + k) * a.nKV + kh) * dv + e] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    if (vo && t0 + k < T) vo[((size_t)(t0 + k) * a.nKV + kh) * dv + e] = (__bf16)x[k];
+    if (vf) x[k] = (1.f - a.v_mix) * x[k] + a.v_mix * m[k];
+  }
+  bool run = slot[0] >= 0 && slot[0] % 8 == 0;
+#pragma unroll
+  for (int k = 1; k < 8; ++k) run = run && slot[k] == slot[0] + k;
+  bf16_t* vc = (bf16_t*)a.v_cache;
+  if (run) {
+    rope_bf16x8 v;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = (__bf16)x[k];
+    const int page = slot[0] / a.page_size, off = slot[0] % a.page_size;
+    *(rope_bf16x8*)(vc + (((size_t)page * a.nKV + kh) * dv + e) * a.page_size + off) = v;
+  } else {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (slot[k] < 0) continue;
+      const int page = slot[k] / a.page_size, off = slot[k] % a.page_size;
+      vc[(((size_t)page * a.nKV + kh) * dv + e) * a.page_size + off] = (__bf16)x[k];
+    }
+  }
+}
+
 // dtype: the type of q_out and the cache, and of qkv unless n_slices > 1 (then qkv holds float partial sums,
 // slice_stride elements apart).
 extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
@@ -608,6 +718,16 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
     const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;
     const unsigned qk_blocks = (unsigned)((qk_threads + 255) / 256), v_blocks = (unsigned)((v_threads + 255) / 256);
     hipLaunchKernelGGL(rope_append_vec_kernel, dim3(qk_blocks + v_blocks), dim3(256), 0, s, a, T, (int)qk_blocks);
+    IFX_LAUNCH_CHECK();
+  }
+  const int rot = rope_style != 0 ? rotary_dim : 0;
+  if (extras && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style <= 1 && (d == 16 || d == 32 || d == 64 || d == 128) &&
+      rot % 16 == 0 && (nH * d + nKV * (d + dv) + gate_cols) % 8 == 0 && (!bias || bias_dtype == DT_BF16) &&
+      (!slots || page_size % 8 == 0) && (slots || (!v_first && !v_out))) {
+    const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
+    const size_t v_threads = (slots || v_out) ? (size_t)((T + 7) / 8) * nKV * dv : 0;
+    const unsigned qk_blocks = (unsigned)((qk_threads + 255) / 256), v_blocks = (unsigned)((v_threads + 255) / 256);
+    hipLaunchKernelGGL(rope_append_vec_x_kernel, dim3(qk_blocks + v_blocks), dim3(256), 0, s, a, T, (int)qk_blocks);
     IFX_LAUNCH_CHECK();
   }
   const dim3 grid(T, nH + 2 * nKV);

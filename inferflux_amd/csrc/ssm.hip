@@ -187,41 +187,65 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
   const T* bc = (const T*)a.bc;
   const T* z = (const T*)a.z;
   float sum_dt = 0.f;
+  // B and C of a token in 8-byte pieces where the sizes allow it (bfloat16, states in fours)
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 scan_bf16x4;
+  const bool pieces = sizeof(T) == 2 && NPT % 4 == 0 && N % 4 == 0 && a.ld_bc % 4 == 0;
+  const int lane0 = (threadIdx.x % WAVE) & ~(LANES - 1);      // the first of the channel's lanes
   for (int i0 = 0; i0 < n_tok; i0 += TOK) {
-    float uv[TOK], dtv[TOK], zv[TOK], Bv[TOK][NPT], Cv[TOK][NPT];
+    float Bv[TOK][NPT], Cv[TOK][NPT];
+    // Of the TOK tokens' inputs that all lanes of a channel need alike (u, the step size, the gate's input) each lane
+    // fetches one token's and forms its step size; the others get them by shuffles (TOK == LANES).
+    static_assert(TOK == LANES, "a channel's lanes take one token each");
+    const size_t t_my = (size_t)t0 + min(i0 + lg, n_tok - 1);
+    const float u_my = to_f(u[t_my * a.C + c]);
+    const float dt_my = softplus_f(a.dt_raw[t_my * a.C + c] + dtb);
+    const float z_my = MODE == 1 ? 0.f : to_f(z[t_my * a.ld_z + c]);
 #pragma unroll
     for (int q = 0; q < TOK; ++q) {
       const bool live = i0 + q < n_tok;
       const size_t t = (size_t)t0 + i0 + (live ? q : 0);
-      uv[q] = to_f(u[t * a.C + c]);
-      dtv[q] = a.dt_raw[t * a.C + c];
-      zv[q] = MODE == 1 ? 0.f : to_f(z[t * a.ld_z + c]);
+      if (pieces) {
 #pragma unroll
-      for (int k = 0; k < NPT; ++k) {
-        const int n = min(n0 + k, N - 1);
-        Bv[q][k] = to_f(bc[t * a.ld_bc + n]);
-        Cv[q][k] = MODE == 1 ? 0.f : to_f(bc[t * a.ld_bc + N + n]);
+        for (int k = 0; k < NPT; k += 4) {
+          const int n = min(n0 + k, N - 4);
+          const scan_bf16x4 b4 = *(const scan_bf16x4*)((const bf16_t*)a.bc + t * a.ld_bc + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) Bv[q][k + e] = (float)b4[e];
+          if (MODE != 1) {
+            const scan_bf16x4 c4 = *(const scan_bf16x4*)((const bf16_t*)a.bc + t * a.ld_bc + N + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Cv[q][k + e] = (float)c4[e];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < NPT; ++k) {
+          const int n = min(n0 + k, N - 1);
+          Bv[q][k] = to_f(bc[t * a.ld_bc + n]);
+          Cv[q][k] = MODE == 1 ? 0.f : to_f(bc[t * a.ld_bc + N + n]);
+        }
       }
     }
 #pragma unroll
     for (int q = 0; q < TOK; ++q) {
+      const float uq = __shfl(u_my, lane0 + q, WAVE), dt = __shfl(dt_my, lane0 + q, WAVE), zq = __shfl(z_my, lane0 + q, WAVE);
       if (i0 + q >= n_tok) break;
-      const float dt = softplus_f(dtv[q] + dtb), dtu = dt * uv[q];
+      const float dtu = dt * uq;
       sum_dt += dt;
       float y = 0.f;
 #pragma unroll
       for (int k = 0; k < NPT; ++k) {
         if (n0 + k < N) {
           S[k] = fmaf(expf(dt * An[k]), S[k], dtu * Bv[q][k]);
-          y = fmaf(S[k], Cv[q][k], y);
+          if (MODE != 1) y = fmaf(S[k], Cv[q][k], y);
         }
       }
       if (MODE != 1) {
         y += __shfl_xor(y, 1, WAVE);      // the channel's four lanes are neighbours
         y += __shfl_xor(y, 2, WAVE);
         if (lg == 0) {
-          y = fmaf(Dc, uv[q], y);
-          ((T*)a.out)[((size_t)t0 + i0 + q) * a.C + c] = from_f<T>(y * act_silu(zv[q]));
+          y = fmaf(Dc, uq, y);
+          ((T*)a.out)[((size_t)t0 + i0 + q) * a.C + c] = from_f<T>(y * act_silu(zq));
         }
       }
     }

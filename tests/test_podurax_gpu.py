@@ -99,10 +99,13 @@ def test_rotation_table_with_stretched_frequencies(dims, base, scaling):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T", [37, 300])       # (many rows of sizes in sixteens take the kernel that works in 16-byte pieces)
 @pytest.mark.parametrize("nH,nKV,d,dv,dims,style", [(4, 2, 16, 24, 8, "mix"), (3, 3, 12, 12, 12, "source"), (2, 1, 32, 8, 4, None),
-                                                    (8, 2, 64, 64, 16, "mix"), (3, 1, 10, 14, 6, "mix"), (5, 5, 130, 70, 100, "source")])
-def test_row_kernel_biases_rotation_unit_norms_gate_value_mixing_and_cache(dtype, nH, nKV, d, dv, dims, style):
-    T, P, pages, eps, lam = 37, 16, 7, 1e-5, 0.3125
+                                                    (8, 2, 64, 64, 16, "mix"), (3, 1, 10, 14, 6, "mix"), (5, 5, 130, 70, 100, "source"),
+                                                    (4, 2, 32, 32, 16, "source"), (8, 8, 128, 128, 64, "mix"), (8, 2, 64, 48, 32, "mix"),
+                                                    (16, 2, 128, 128, 128, None), (8, 1, 16, 16, 16, "mix")])
+def test_row_kernel_biases_rotation_unit_norms_gate_value_mixing_and_cache(dtype, T, nH, nKV, d, dv, dims, style):
+    P, pages, eps, lam = 16, -(-T // 16) + 4, 1e-5, 0.3125
     dt = DT[dtype]
     width = (nH + nKV) * d + nKV * dv + nH
     qkv, bias = rnd(1, T, width, scale=1.5).to(dt), rnd(2, width, scale=0.5).to(dt)
@@ -121,7 +124,8 @@ def test_row_kernel_biases_rotation_unit_norms_gate_value_mixing_and_cache(dtype
                         v_first.to(DEV) if style == "mix" else None, lam, v_out)
     x = (qkv.double() + bias.double()).numpy()
     pos = positions.numpy()
-    tol = 1e-5 if dtype == "float32" else 1e-2
+    # (32-bit: the engine forms angles in float, position times frequency, which at position p is off by up to p * 6e-8)
+    tol = 1e-5 + 1e-7 * int(positions.max()) if dtype == "float32" else 1e-2
     want_q = pp.rms(pp.rotate(x[:, :nH * d].reshape(T, nH, d), pos, dims, 1000.0, sc), eps)
     assert rel_err(q.cpu(), T64(want_q)) < tol
     want_k = pp.rms(pp.rotate(x[:, nH * d:(nH + nKV) * d].reshape(T, nKV, d), pos, dims, 1000.0, sc), eps)
