@@ -420,6 +420,34 @@ def test_whole_prompts(name, dtype, folders):
     runner.manager.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["recurrent_only", "no_windows", "one_attention"])
+def test_models_without_pages_or_without_windows(kind, dtype, tmp_path):
+    """A model of recurrences alone keeps no pages at all; attention without a window keeps everything (kept first tokens
+    then mean nothing); a single attention layer that mixes values has nobody to mix with."""
+    layers = {
+        "recurrent_only": [pm.layer(pm.mamba1(48, 8, 4, 3), 40), pm.layer(pm.mamba1(32, 3, 2, 4), None)],
+        "no_windows": [pm.layer(pm.attention(4, 1, 16, 16, 0.5, 10000.0, 16, window=None, keep_first=9), 40),
+                       pm.layer(pm.attention(2, 2, 32, 16, 0.4, 500.0, 8, v_mix=False), 24)],
+        "one_attention": [pm.layer(pm.attention(4, 4, 64, 64, 0.2, 1e6, 16, window=96, keep_first=6, scaling=(8.0, 1024, 32.0, 1.0)), 64)],
+    }[kind]
+    cfg = pm.model(150, 64, 1e-5, 0.5, 0.5, layers)
+    folder = pm.write_model(str(tmp_path / "m"), cfg, 9, gain=GAIN[dtype])
+    runner = load_runner(folder, DT[dtype], num_pages=20, max_requests=3)
+    assert len(runner.manager.groups) == {"recurrent_only": 0, "no_windows": 1, "one_attention": 1}[kind]
+    ids = ids_of(8, 230, 150)
+    want = plain(folder, ids)
+    assert rel_err(run_whole(runner, "w", ids), want) < TOL[dtype]
+    runner.add_request("c")
+    runner.add_request("o")
+    rows, p = [], 0
+    for m in [2, 100, 1, 1, 64, 3, 1, 58]:
+        rows.append(runner.step([StepEntry("o", ids_of(p, 2, 150), []), StepEntry("c", ids[p:p + m], list(range(m)))]).cpu())
+        p += m
+    assert p == len(ids) and rel_err(torch.cat(rows), want) < TOL[dtype]
+    runner.manager.check()
+
+
 @pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_stream_after_every_layer(name, folders):
     folder = folders[name, "float32"]
