@@ -131,7 +131,8 @@ __device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& 
   }
 }
 
-template <bool STREAM>
+// KEEP: the launch has kept first keys (a.keep_first > 0); without them the walk below is the plain one, at its old cost.
+template <bool STREAM, bool KEEP>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_rows_kernel(RowArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, ri = blockIdx.z;
   const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
@@ -148,9 +149,9 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
   // ... and of the kept first keys [0, keep) those of this split: [split * chunk, ke).  Where there are any the walk
   // starts at the split's first key and passes whatever lies between them and the window without loading it.
-  const int keep = lo > 0 ? min(a.keep_first, lo) : 0;
-  const int ke = split * a.chunk < keep ? min(keep, min(pos + 1, (split + 1) * a.chunk)) : 0;
-  const int walk0 = ke > 0 ? split * a.chunk : ka;
+  const int keep = (KEEP && lo > 0) ? min(a.keep_first, lo) : 0;
+  const int ke = (KEEP && split * a.chunk < keep) ? min(keep, min(pos + 1, (split + 1) * a.chunk)) : 0;
+  const int walk0 = (KEEP && ke > 0) ? split * a.chunk : ka;
   const int ratio = a.nH / a.nKV;
   const int* table = early ? early_table : a.block_table + (size_t)a.row_req[row] * a.max_blocks;
 
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 // Dynamic LDS: waves x nc x (D + 4) floats of outputs and waves x nc x 2 of (max, sum); nc = heads per pass.
 constexpr int OPAD = D + 4;       // floats per output row in LDS (the padding spreads the 16 columns over the banks)
 
-template <bool STREAM>
+template <bool STREAM, bool KEEP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_rows_whole_kernel(RowArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int kvh = blockIdx.x, ri = blockIdx.y;
@@ -240,15 +241,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // kept first keys [0, keep) before the window the runs are numbered as if the window's first run followed the last
   // kept run: walk place v is key v below kr and key v + gap from there on.
   const int first = lo / 32 * 32;
-  const int keep = lo > 0 ? min(a.keep_first, lo) : 0;
+  const int keep = (KEEP && lo > 0) ? min(a.keep_first, lo) : 0;
   const int keep_runs = (keep + 31) / 32 * 32;
-  const int base = keep > 0 ? 0 : first;
-  const int gap = (keep > 0 && keep_runs < first) ? first - keep_runs : 0, kr = gap > 0 ? keep_runs : 0;
+  const int base = (KEEP && keep > 0) ? 0 : first;
+  const int gap = (KEEP && keep > 0 && keep_runs < first) ? first - keep_runs : 0, kr = (KEEP && gap > 0) ? keep_runs : 0;
   const int vend = pos + 1 - gap;
   const int chunk = ((vend - base + W - 1) / W + 31) / 32 * 32;
   const int va = base + wid * chunk, vb = min(vend, base + (wid + 1) * chunk);     // this wave's places [va, vb), whole runs
   const int ka = lo, kb = pos + 1, ke = keep;                                      // what is visible at all
-  auto key_at = [&](int v) { return v < kr ? v : v + gap; };
+  auto key_at = [&](int v) { return KEEP ? (v < kr ? v : v + gap) : v; };
   const int ratio = a.nH / a.nKV;
   const int nc_max = min(16, ratio);
   const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
@@ -359,16 +360,24 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
     const int nc = nH / nKV < 16 ? nH / nKV : 16;
     const size_t lds = (size_t)waves * nc * (OPAD + 2) * sizeof(float);
     IFX_REQUIRE(lds <= 65536, "attn_rows: %d waves of %d heads need %zu bytes of LDS", waves, nc, lds);
-    if (streaming)
-      hipLaunchKernelGGL(attn_rows_whole_kernel<true>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
-    else
-      hipLaunchKernelGGL(attn_rows_whole_kernel<false>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+    if (a.keep_first > 0) {
+      if (streaming) hipLaunchKernelGGL((attn_rows_whole_kernel<true, true>), dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+      else hipLaunchKernelGGL((attn_rows_whole_kernel<false, true>), dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+    } else {
+      if (streaming) hipLaunchKernelGGL((attn_rows_whole_kernel<true, false>), dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+      else hipLaunchKernelGGL((attn_rows_whole_kernel<false, false>), dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+    }
     IFX_LAUNCH_CHECK();
   }
   IFX_REQUIRE(chunk > 0 && chunk % 32 == 0 && max_splits > 0 && max_splits <= 65535, "attn_rows: bad chunk %d / splits %d", chunk, max_splits);
   IFX_REQUIRE(part_o && part_ml, "attn_rows: splits need scratch for their partial results");
-  if (streaming) hipLaunchKernelGGL(attn_rows_kernel<true>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
-  else hipLaunchKernelGGL(attn_rows_kernel<false>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+  if (a.keep_first > 0) {
+    if (streaming) hipLaunchKernelGGL((attn_rows_kernel<true, true>), dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+    else hipLaunchKernelGGL((attn_rows_kernel<false, true>), dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+  } else {
+    if (streaming) hipLaunchKernelGGL((attn_rows_kernel<true, false>), dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+    else hipLaunchKernelGGL((attn_rows_kernel<false, false>), dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+  }
   hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, a);
   IFX_LAUNCH_CHECK();
 }
