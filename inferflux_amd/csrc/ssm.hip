@@ -52,6 +52,54 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
   ((T*)a.out)[(size_t)t * a.C + c] = from_f<T>(act_silu(acc));
 }
 
+// The same for bfloat16 rows with channels in eights and TAPS taps (known at compile time, so that every index below is):
+// a thread takes eight neighbouring channels of one token, every tap's inputs as one 16-byte piece, the eight channels'
+// weights as TAPS such pieces.  The sums are formed in the same order.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 conv_bf16x8;
+
+template <int TAPS>
+__global__ __launch_bounds__(256) void conv_silu_vec_kernel(ConvArgs a) {
+  const int c = 8 * (blockIdx.x * 256 + threadIdx.x), t = blockIdx.y;
+  if (c >= a.C) return;
+  const int r = a.row_req[t], t0 = a.q_start[r], i = t - t0;
+  const bf16_t* x = (const bf16_t*)a.x;
+  conv_bf16x8 wv[TAPS], xv[TAPS];       // weights [8 channels][TAPS] as one run; inputs of tap j for the eight channels
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) wv[j] = *(const conv_bf16x8*)((const bf16_t*)a.w + (size_t)c * TAPS + 8 * j);
+  float acc[8];
+  if (a.b) {
+    const conv_bf16x8 b8 = *(const conv_bf16x8*)((const bf16_t*)a.b + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = (float)b8[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  }
+  if (i >= TAPS - 1) {       // every input is a row of this step: the usual case
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) xv[j] = *(const conv_bf16x8*)(x + (size_t)(t - (TAPS - 1) + j) * a.ld + c);
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf((float)wv[(e * TAPS + j) / 8][(e * TAPS + j) % 8], (float)xv[j][e], acc[e]);
+  } else {
+    const float* st = a.state + (size_t)a.slots[r] * a.state_stride + (size_t)c * (TAPS - 1);
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int src = i - (TAPS - 1) + j;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float in = src >= 0 ? (float)x[(size_t)(t0 + src) * a.ld + c + e] : st[(size_t)e * (TAPS - 1) + src + TAPS - 1];
+        acc[e] = fmaf((float)wv[(e * TAPS + j) / 8][(e * TAPS + j) % 8], in, acc[e]);
+      }
+    }
+  }
+  conv_bf16x8 y;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = (__bf16)act_silu(acc[e]);
+  *(conv_bf16x8*)((bf16_t*)a.out + (size_t)t * a.C + c) = y;
+}
+
 // After the convolution has read the slots: every request's last taps - 1 inputs, from this step's rows and, where
 // the step brought fewer, from what the slot held.  One thread owns a (request, channel): it reads before it writes.
 template <typename T>
@@ -90,7 +138,14 @@ extern "C" int ifx_causal_conv(const void* x, int dtype, int ld, const void* w, 
     hipLaunchKernelGGL(conv_silu_kernel<float>, dim3(cb, T), dim3(256), 0, s, a);
     if (taps > 1) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(cb, R), dim3(256), 0, s, a);
   } else if (dtype == DT_BF16) {
-    hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, dim3(cb, T), dim3(256), 0, s, a);
+    // (many rows only: a thread of eight channels leaves a step of few rows too few threads to fill the chip)
+    const bool vec = C % 8 == 0 && ld % 8 == 0 && w_dtype == DT_BF16 && (long long)T * C >= (1 << 20);
+    const dim3 vgrid((unsigned)((C / 8 + 255) / 256), T);
+    if (vec && taps == 4) hipLaunchKernelGGL(conv_silu_vec_kernel<4>, vgrid, dim3(256), 0, s, a);
+    else if (vec && taps == 3) hipLaunchKernelGGL(conv_silu_vec_kernel<3>, vgrid, dim3(256), 0, s, a);
+    else if (vec && taps == 2) hipLaunchKernelGGL(conv_silu_vec_kernel<2>, vgrid, dim3(256), 0, s, a);
+    else
+      hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, dim3(cb, T), dim3(256), 0, s, a);
     if (taps > 1) hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(cb, R), dim3(256), 0, s, a);
   } else IFX_FAIL("causal_conv: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
@@ -118,6 +173,10 @@ struct ScanArgs {
 };
 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// exp of a decay's exponent (<= 0).  With bfloat16 activations the hardware's 2^x (about two units in the last place of a
+// float; a token's y is rounded to 8 bits of mantissa afterwards); in 32-bit the library's.
+template <typename T> __device__ __forceinline__ float decay(float x) { return sizeof(T) == 2 ? __expf(x) : expf(x); }
 
 // LANES lanes share a channel, each with NPT of its states (state n belongs to lane n / NPT); a token's sum over the
 // states is added across them in a fixed order.  TOK tokens' inputs are asked for together, so that the recurrence,
@@ -236,7 +295,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
 #pragma unroll
       for (int k = 0; k < NPT; ++k) {
         if (n0 + k < N) {
-          S[k] = fmaf(expf(dt * An[k]), S[k], dtu * Bv[q][k]);
+          S[k] = fmaf(decay<T>(dt * An[k]), S[k], dtu * Bv[q][k]);
           if (MODE != 1) y = fmaf(S[k], Cv[q][k], y);
         }
       }

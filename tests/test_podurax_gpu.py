@@ -297,6 +297,28 @@ def test_causal_convolution_carries_its_last_inputs_from_step_to_step(dtype, C, 
     assert torch.all(state[1] == 7.0) and torch.all(state[:, C * (taps - 1):][[0, 2, 3]] == 0)
 
 
+@pytest.mark.parametrize("taps", [2, 3, 4, 5])
+def test_causal_convolution_of_many_rows(taps):
+    """Steps of many rows in bfloat16 take the kernel that works in 16-byte pieces (2 to 4 taps): two requests, the second
+    continued from its slot, then single rows behind them."""
+    C, lens = 2048, [[300, 260], [270, 1], [1, 2]]
+    totals = [sum(step[i] for step in lens) for i in range(2)]
+    xs = [rnd(80 + i, n, 2 * C).to(torch.bfloat16) for i, n in enumerate(totals)]
+    w, b = rnd(82, C, taps, scale=0.6).to(torch.bfloat16), rnd(83, C, scale=0.3).to(torch.bfloat16)
+    state = torch.zeros((3, C * (taps - 1)), dtype=torch.float32, device=DEV)
+    slots = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+    got, at = [[], []], [0, 0]
+    for step in lens:
+        x = torch.cat([xs[i][at[i]:at[i] + step[i]] for i in range(2)])
+        q_start, q_len, row_req = _step_arrays(step)
+        out = ops.causal_conv_silu(x.to(DEV), C, w.to(DEV), b.to(DEV), state, row_req.to(DEV), q_start.to(DEV), q_len.to(DEV), slots).cpu()
+        got[0].append(out[:step[0]]); got[1].append(out[step[0]:])
+        at = [at[i] + step[i] for i in range(2)]
+    for i in range(2):
+        want = pp.silu(pp.causal_conv(xs[i].double().numpy()[:, :C], w.double().numpy(), b.double().numpy()))
+        assert rel_err(torch.cat(got[i]), T64(want)) < 1e-2, i
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("C,N", [(96, 6), (40, 17), (56, 4), (256, 16), (50, 5), (24, 1), (32, 33), (16, 128)])
 def test_selective_scan_carries_its_state_from_step_to_step(dtype, C, N):
