@@ -80,7 +80,7 @@ DESIGN_SIZES = {
 # repeated to the depth: the sizes with one kind alone say what each mechanism costs.
 def _podurax_shape(width, layers, heads, kv_heads, dim, window, ff, inner, state, dt_rank, pattern, vocab=32000):
     att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5 * 8.0, "v_mix": True,
-           "rot": {"base": 1e6, "dims": dim // 2, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+           "rot": {"base": 5e5, "dims": dim // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 1.0}},
            "mask": {"size": window, "keep_first": 4}}
     ssm = {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": 4}
     mix = {"a": ("attention", att), "m": ("mamba1", ssm)}

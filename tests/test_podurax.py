@@ -170,16 +170,16 @@ def test_sink_softmax_is_a_softmax_over_the_keys_and_a_zero():
 
 
 def test_stretched_frequencies_keep_the_fast_pairs_and_stretch_the_slow():
-    f, mag = pp.yarn_frequencies(16, 1e6, {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0})
-    plain_f, one = pp.yarn_frequencies(16, 1e6, None)
-    assert one == 1.0 and np.allclose(plain_f, [1e6 ** (-2 * i / 16) for i in range(8)])
-    assert np.isclose(mag, 0.1 * math.log(8.0) + 1.0)
-    assert np.allclose(f[0], plain_f[0]) and np.allclose(f[-1], plain_f[-1] / 8.0)          # the ends of the ramp
-    assert all(b / 8.0 - 1e-18 <= a <= b + 1e-18 for a, b in zip(f, plain_f)) and list(f) == sorted(f, reverse=True)
-    x = np.random.default_rng(1).normal(size=(3, 2, 20))
-    y = pp.rotate(x, np.array([0, 5, 900]), 16, 1e6, {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0})
-    assert np.allclose(y[..., 16:], x[..., 16:])                                             # the rest passes unchanged
-    assert np.allclose((y[..., :16] ** 2).sum(-1), mag ** 2 * (x[..., :16] ** 2).sum(-1))    # a rotation, lengthened by the factor
+    f, mag = pp.yarn_frequencies(24, 5e5, {"factor": 6.0, "original": 2048, "fast": 24.0, "slow": 1.0})
+    plain_f, one = pp.yarn_frequencies(24, 5e5, None)
+    assert one == 1.0 and np.allclose(plain_f, [5e5 ** (-2 * i / 24) for i in range(12)])
+    assert np.isclose(mag, 0.1 * math.log(6.0) + 1.0)
+    assert np.allclose(f[0], plain_f[0]) and np.allclose(f[-1], plain_f[-1] / 6.0)          # the ends of the ramp
+    assert all(b / 6.0 - 1e-18 <= a <= b + 1e-18 for a, b in zip(f, plain_f)) and list(f) == sorted(f, reverse=True)
+    x = np.random.default_rng(1).normal(size=(3, 2, 30))
+    y = pp.rotate(x, np.array([0, 5, 900]), 24, 5e5, {"factor": 6.0, "original": 2048, "fast": 24.0, "slow": 1.0})
+    assert np.allclose(y[..., 24:], x[..., 24:])                                             # the rest passes unchanged
+    assert np.allclose((y[..., :24] ** 2).sum(-1), mag ** 2 * (x[..., :24] ** 2).sum(-1))    # a rotation, lengthened by the factor
 
 
 def test_the_recurrence_cut_anywhere_carries_on_from_its_state():
