@@ -55,6 +55,14 @@ CONFIGS = {
         layer(mamba1(256, 16, 8, 4), 192),
         layer(attention(8, 2, 32, 64, 0.3, 10000.0, 16, window=48, keep_first=4), 128),
     ]),
+    # a size at which the products take their other kernels (weights in tiles, K in slices, the library for prompts), heads of
+    # 96 and 48, a recurrence of 1,024 channels
+    "E": model(1000, 512, 1e-5, 1.0, 0.6, [
+        layer(attention(8, 2, 96, 96, 0.12, 50000.0, 32, window=128, keep_first=8, scaling=(4.0, 512, 16.0, 2.0)), 1536),
+        layer(mamba1(1024, 16, 32, 4), 1536),
+        layer(attention(16, 2, 48, 96, 0.2, 50000.0, 48, window=40, keep_first=2), None),
+        layer(mamba1(768, 8, 24, 3), 1024),
+    ]),
     # nothing a multiple of 8; more kept first tokens than the window is long, and nearly as many
     "D": model(99, 100, 1e-5, 1.5, 0.8, [
         layer(attention(3, 1, 10, 14, 0.9, 3000.0, 6, window=9, keep_first=40), 50),

@@ -499,7 +499,7 @@ def test_first_tokens(folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "D", "E"])
 def test_prefill_against_decoding_and_portions(name, dtype, folders):
     folder, vocab = folders[name, dtype], pm.CONFIGS[name]["vocab"]
     runner = load_runner(folder, DT[dtype], num_pages=24, max_requests=4)
@@ -627,7 +627,9 @@ def _drawn_config(seed):
             mixer = pm.mamba1(rng.choice([24, 64, 100, 192]), rng.choice([1, 4, 7, 16, 24]), rng.choice([1, 4, 8, 10]), rng.choice([1, 2, 4, 5]))
         else:
             kv = rng.choice([1, 2, 3])
-            dim, vdim = rng.choice([8, 12, 16, 32, 64]), rng.choice([8, 10, 16, 32, 64])
+            dim, vdim = rng.choice([8, 12, 16, 32, 48, 64, 96, 128]), rng.choice([8, 10, 16, 32, 64])
+            if rng.random() < 0.5:
+                vdim = dim                                  # (values as wide as keys: the matrix-core kernels where the size allows)
             v_mix = rng.random() < 0.7
             if v_mix:
                 mixing = mixing or (kv, vdim)
@@ -641,7 +643,7 @@ def _drawn_config(seed):
     return pm.model(rng.choice([61, 128, 500]), width, rng.choice([1e-5, 1e-6, 1e-3]), rng.choice([1.0, 0.5, 3.0]), rng.choice([1.0, 0.5, 0.3]), layers)
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(14))
 def test_drawn_configurations(seed, tmp_path):
     """Whole prompts, portions and decoding of drawn configurations against the plain implementation, both precisions."""
     cfg = _drawn_config(seed)
