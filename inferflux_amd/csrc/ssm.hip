@@ -204,9 +204,12 @@ struct ChunkArgs {
 
 template <typename T, int NPT, int MODE>
 __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char scan_lds[];       // modes 1 and 3: the chunk's B and C rows
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  const int c = idx / LANES, lg = idx % LANES;
-  if (c >= a.C) return;          // (C * LANES is a multiple of LANES: the lanes of a channel leave together)
+  const int c_raw = idx / LANES, lg = idx % LANES;
+  const bool active = c_raw < a.C;      // (the lanes of a channel are active together; in modes 1 and 3 nobody leaves before the barrier)
+  if ((MODE == 0 || MODE == 2) && !active) return;
+  const int c = active ? c_raw : a.C - 1;
   const int N = a.N, n0 = lg * NPT;
   float An[NPT];
 #pragma unroll
@@ -246,9 +249,21 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
   const T* bc = (const T*)a.bc;
   const T* z = (const T*)a.z;
   float sum_dt = 0.f;
+  // Modes 1 and 3: a chunk's B and C are the same for every channel; the workgroup copies them into LDS once (rows of
+  // 2 N, the chunk's first row first) and the walk below reads them there instead of from memory.
+  constexpr bool STAGED = MODE == 1 || MODE == 3;
+  T* bc_s = (T*)scan_lds;
+  if (STAGED) {
+    const int per_row = 2 * N, total = n_tok * per_row;
+    for (int i = threadIdx.x; i < total; i += 256) bc_s[i] = bc[(size_t)(t0 + i / per_row) * a.ld_bc + i % per_row];
+    __syncthreads();
+    if (!active) return;
+  }
+  const T* bc_rows = STAGED ? bc_s : bc + (size_t)t0 * a.ld_bc;        // row i of the walk starts at bc_rows + i * bc_ld
+  const int bc_ld = STAGED ? 2 * N : a.ld_bc;
   // B and C of a token in 8-byte pieces where the sizes allow it (bfloat16, states in fours)
   typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 scan_bf16x4;
-  const bool pieces = sizeof(T) == 2 && NPT % 4 == 0 && N % 4 == 0 && a.ld_bc % 4 == 0;
+  const bool pieces = sizeof(T) == 2 && NPT % 4 == 0 && N % 4 == 0 && bc_ld % 4 == 0;
   const int lane0 = (threadIdx.x % WAVE) & ~(LANES - 1);      // the first of the channel's lanes
   for (int i0 = 0; i0 < n_tok; i0 += TOK) {
     float Bv[TOK][NPT], Cv[TOK][NPT];
@@ -262,16 +277,16 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
 #pragma unroll
     for (int q = 0; q < TOK; ++q) {
       const bool live = i0 + q < n_tok;
-      const size_t t = (size_t)t0 + i0 + (live ? q : 0);
+      const T* row = bc_rows + (size_t)(i0 + (live ? q : 0)) * bc_ld;
       if (pieces) {
 #pragma unroll
         for (int k = 0; k < NPT; k += 4) {
           const int n = min(n0 + k, N - 4);
-          const scan_bf16x4 b4 = *(const scan_bf16x4*)((const bf16_t*)a.bc + t * a.ld_bc + n);
+          const scan_bf16x4 b4 = *(const scan_bf16x4*)((const bf16_t*)row + n);
 #pragma unroll
           for (int e = 0; e < 4; ++e) Bv[q][k + e] = (float)b4[e];
           if (MODE != 1) {
-            const scan_bf16x4 c4 = *(const scan_bf16x4*)((const bf16_t*)a.bc + t * a.ld_bc + N + n);
+            const scan_bf16x4 c4 = *(const scan_bf16x4*)((const bf16_t*)row + N + n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) Cv[q][k + e] = (float)c4[e];
           }
@@ -280,8 +295,8 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
 #pragma unroll
         for (int k = 0; k < NPT; ++k) {
           const int n = min(n0 + k, N - 1);
-          Bv[q][k] = to_f(bc[t * a.ld_bc + n]);
-          Cv[q][k] = MODE == 1 ? 0.f : to_f(bc[t * a.ld_bc + N + n]);
+          Bv[q][k] = to_f(row[n]);
+          Cv[q][k] = MODE == 1 ? 0.f : to_f(row[N + n]);
         }
       }
     }
@@ -317,7 +332,10 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs a, ChunkArgs ch) {
 }
 
 template <typename T>
-static int launch_scan(const ScanArgs& a, const ChunkArgs& ch, int n_chunks, hipStream_t s) {
+static int launch_scan(const ScanArgs& a, const ChunkArgs& ch, int n_chunks, int max_chunk, hipStream_t s) {
+  const size_t lds = (size_t)max_chunk * 2 * a.N * sizeof(T);      // a chunk's B and C rows
+  IFX_REQUIRE(n_chunks <= 0 || (max_chunk > 0 && lds <= 64 * 1024), "selective_scan: chunks of %d rows x %d states need %zu bytes of LDS",
+              max_chunk, a.N, lds);
   const int npt = (a.N + LANES - 1) / LANES;
   const unsigned gx = (unsigned)(((size_t)a.C * LANES + 255) / 256);
   const dim3 grid(gx, a.R), grid_chunks(gx, n_chunks > 0 ? n_chunks : 1);
@@ -325,9 +343,9 @@ static int launch_scan(const ScanArgs& a, const ChunkArgs& ch, int n_chunks, hip
   do {                                                                                            \
     if (n_chunks <= 0) hipLaunchKernelGGL((scan_kernel<T, NPT_, 0>), grid, dim3(256), 0, s, a, ch); \
     else {                                                                                        \
-      hipLaunchKernelGGL((scan_kernel<T, NPT_, 1>), grid_chunks, dim3(256), 0, s, a, ch);         \
+      hipLaunchKernelGGL((scan_kernel<T, NPT_, 1>), grid_chunks, dim3(256), lds, s, a, ch);         \
       hipLaunchKernelGGL((scan_kernel<T, NPT_, 2>), grid, dim3(256), 0, s, a, ch);                \
-      hipLaunchKernelGGL((scan_kernel<T, NPT_, 3>), grid_chunks, dim3(256), 0, s, a, ch);         \
+      hipLaunchKernelGGL((scan_kernel<T, NPT_, 3>), grid_chunks, dim3(256), lds, s, a, ch);         \
     }                                                                                             \
   } while (0)
   if (npt <= 1) GO(1);
@@ -347,7 +365,7 @@ extern "C" int ifx_selective_scan(const void* u, int dtype, const float* dt_raw,
                                   const void* bc, int ld_bc, const void* D, int w_dtype, const void* z, int ld_z,
                                   float* state, long long state_stride, long long state_offset, const int* q_start,
                                   const int* q_len, const int* slots, void* out, int T, int R, int C, int N,
-                                  int n_chunks, const int* chunk_req, const int* chunk_t0, const int* chunk_len,
+                                  int n_chunks, int max_chunk, const int* chunk_req, const int* chunk_t0, const int* chunk_len,
                                   const int* req_chunk0, float* chunk_state, float* chunk_dt, void* stream) {
   IFX_REQUIRE(n_chunks >= 0 && n_chunks <= 65535, "selective_scan: %d chunks", n_chunks);
   IFX_REQUIRE(n_chunks == 0 || (chunk_req && chunk_t0 && chunk_len && req_chunk0 && chunk_state && chunk_dt),
@@ -360,7 +378,7 @@ extern "C" int ifx_selective_scan(const void* u, int dtype, const float* dt_raw,
   ScanArgs a{u, dt_raw, dt_bias, A, bc, ld_bc, D, w_dtype, z, ld_z, state, (size_t)state_stride, (size_t)state_offset,
              q_start, q_len, slots, out, R, C, N};
   const ChunkArgs ch{chunk_req, chunk_t0, chunk_len, req_chunk0, chunk_state, chunk_dt};
-  if (dtype == DT_F32) return launch_scan<float>(a, ch, n_chunks, (hipStream_t)stream);
-  if (dtype == DT_BF16) return launch_scan<bf16_t>(a, ch, n_chunks, (hipStream_t)stream);
+  if (dtype == DT_F32) return launch_scan<float>(a, ch, n_chunks, max_chunk, (hipStream_t)stream);
+  if (dtype == DT_BF16) return launch_scan<bf16_t>(a, ch, n_chunks, max_chunk, (hipStream_t)stream);
   IFX_FAIL("selective_scan: unknown dtype %d", dtype);
 }

@@ -1095,7 +1095,7 @@ def causal_conv_silu(x: torch.Tensor, channels: int, weight: torch.Tensor, bias:
 
 def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, bc: torch.Tensor,
                    D: torch.Tensor, z: torch.Tensor, state: torch.Tensor, state_offset: int, q_start: torch.Tensor,
-                   q_len: torch.Tensor, slots: torch.Tensor, chunks: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
+                   q_len: torch.Tensor, slots: torch.Tensor, chunks: Optional[Dict[str, object]] = None) -> torch.Tensor:
     """The recurrence of a selective state-space mixer over each request's rows, then the gate:
     dt = softplus(dt_raw + dt_bias); S[c, n] <- exp(dt A[c, n]) S[c, n] + dt u[c] B[n]; y[c] = sum_n S[c, n] C[n] + D[c] u[c];
     out = y * silu(z).  ``u`` [T, C], ``dt_raw`` float32 [T, C], ``A`` float32 [C, N] (negative), ``bc`` [T, >= 2N] with B
@@ -1120,9 +1120,9 @@ def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
     for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
         _check(t, nm, (R,), torch.int32)
     out = torch.empty((T, C), dtype=u.dtype, device=u.device)
-    n_chunks, lists = 0, (0, 0, 0, 0, 0, 0)
+    n_chunks, max_chunk, lists = 0, 0, (0, 0, 0, 0, 0, 0)
     if chunks is not None:
-        n_chunks = chunks["req"].shape[0]
+        n_chunks, max_chunk = chunks["req"].shape[0], int(chunks["rows"])
         for nm in ("req", "t0", "len"):
             _check(chunks[nm], f"chunks.{nm}", (n_chunks,), torch.int32)
         _check(chunks["req_chunk0"], "chunks.req_chunk0", (R + 1,), torch.int32)
@@ -1131,14 +1131,14 @@ def selective_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
         lists = (chunks["req"].data_ptr(), chunks["t0"].data_ptr(), chunks["len"].data_ptr(), chunks["req_chunk0"].data_ptr(),
                  chunk_state.data_ptr(), chunk_dt.data_ptr())
     _call(load_module("ssm"), "ifx_selective_scan",
-          (P, I, P, P, P, P, I, P, I, P, I, P, LL, LL, P, P, P, P, I, I, I, I, I, P, P, P, P, P, P, P),
+          (P, I, P, P, P, P, I, P, I, P, I, P, LL, LL, P, P, P, P, I, I, I, I, I, I, P, P, P, P, P, P, P),
           u.data_ptr(), _dt(u), dt_raw.data_ptr(), dt_bias.data_ptr(), A.data_ptr(), bc.data_ptr(), bc.shape[1], D.data_ptr(),
           _dt(D), z.data_ptr(), z.stride(0) if T else C, state.data_ptr(), state.shape[1], int(state_offset), q_start.data_ptr(),
-          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, C, N, n_chunks, *lists, _stream())
+          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, C, N, n_chunks, max_chunk, *lists, _stream())
     return out
 
 
-def scan_chunks(q_start, q_len, chunk: int, device) -> Dict[str, torch.Tensor]:
+def scan_chunks(q_start, q_len, chunk: int, device) -> Dict[str, object]:
     """The lists ``selective_scan`` takes as ``chunks``: every request's rows (host arrays ``q_start`` / ``q_len`` of the
     step) cut into chunks of up to ``chunk`` rows, in one upload."""
     import numpy as np
@@ -1151,7 +1151,8 @@ def scan_chunks(q_start, q_len, chunk: int, device) -> Dict[str, torch.Tensor]:
     pad = lambda v: v + [0] * (-len(v) % 4)
     packed = torch.from_numpy(np.asarray(pad(req) + pad(t0) + pad(ln) + first, dtype=np.int32)).to(device)
     w = n + -n % 4
-    return {"req": packed[:n], "t0": packed[w:w + n], "len": packed[2 * w:2 * w + n], "req_chunk0": packed[3 * w:3 * w + len(first)]}
+    return {"req": packed[:n], "t0": packed[w:w + n], "len": packed[2 * w:2 * w + n], "req_chunk0": packed[3 * w:3 * w + len(first)],
+            "rows": int(chunk)}       # (the most rows a chunk has: the kernels keep a chunk's B and C in LDS)
 
 
 WIDE_MAX_K_DIM, WIDE_MAX_V_DIM = 1024, 512
