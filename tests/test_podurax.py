@@ -223,3 +223,26 @@ def test_the_whole_model_changes_when_a_mechanism_is_left_out(tmp_path):
     W2 = dict(W)
     W2["l1.mix.A_log"] = W["l1.mix.A_log"] + 0.5
     assert np.abs(pp.forward(cfg, W2, ids) - base).max() / scale > 1e-3
+
+
+def test_random_weights_folder_roundtrips_with_its_scalar_tensors(tmp_path):
+    """The seeded random-weights mode writes every tensor the plan declares, the scalar mixing weights among them, with
+    decays and step-size biases in the range a recurrence needs; the folder reads back equal and its config reloads."""
+    import torch
+    from safetensors.torch import load_file
+    from inferflux_amd.weights import write_random_model
+    from inferflux_amd.weights.safetensors_io import open_model_files
+    cfg = config_from_dict(pm.config("A"))
+    folder = str(tmp_path / "m")
+    write_random_model(folder, cfg, seed=3)
+    assert load_config(folder) == cfg
+    t = load_file(folder + "/model.safetensors")
+    assert set(t) == set(Model(cfg).param_specs())
+    assert t["l0.mix.vmix"].shape == () and 0.2 <= float(t["l2.mix.vmix"]) <= 0.8
+    assert float(t["l1.mix.A_log"].float().exp().min()) >= 0.99 and float(t["l1.mix.dt.b"].float().max()) <= -0.99
+    files = open_model_files(folder)
+    mine = files[0].tensor("l2.mix.vmix") if hasattr(files[0], "tensor") else None
+    if mine is not None:
+        assert torch.equal(mine, t["l2.mix.vmix"])
+    write_random_model(str(tmp_path / "again"), cfg, seed=3)
+    assert all(torch.equal(v, load_file(str(tmp_path / "again") + "/model.safetensors")[k]) for k, v in t.items())

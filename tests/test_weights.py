@@ -16,7 +16,8 @@ def test_container_roundtrip_against_the_safetensors_package(tmp_path):
     from safetensors.torch import load_file, save_file
     g = torch.Generator().manual_seed(0)
     tensors = {"a": torch.randn(3, 5, generator=g).bfloat16(), "b.c": torch.randn(7, generator=g),
-               "i": torch.arange(6, dtype=torch.int32).view(2, 3), "h": torch.randn(2, 2, generator=g).half()}
+               "i": torch.arange(6, dtype=torch.int32).view(2, 3), "h": torch.randn(2, 2, generator=g).half(),
+               "scalar": torch.tensor(0.375).bfloat16()}
     ours = str(tmp_path / "ours.safetensors")
     write_safetensors(ours, tensors, metadata={"format": "pt"})
     theirs = load_file(ours)                       # the independent reader accepts what we write
