@@ -57,15 +57,24 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
 // weights as TAPS such pieces.  The sums are formed in the same order.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 conv_bf16x8;
 
+// A workgroup is CONV_WG_ROWS consecutive rows by 256 / CONV_WG_ROWS threads of eight channels: a row that is an input of
+// TAPS outputs is fetched from memory by one of them and found in the compute unit's cache by the others.
+constexpr int CONV_WG_ROWS = 8;
+
 template <int TAPS>
 __global__ __launch_bounds__(256) void conv_silu_vec_kernel(ConvArgs a) {
-  const int c = 8 * (blockIdx.x * 256 + threadIdx.x), t = blockIdx.y;
-  if (c >= a.C) return;
-  const int r = a.row_req[t], t0 = a.q_start[r], i = t - t0;
+  constexpr int WG_COLS = 256 / CONV_WG_ROWS;
+  const int c = 8 * (blockIdx.x * WG_COLS + threadIdx.x % WG_COLS), t = blockIdx.y * CONV_WG_ROWS + threadIdx.x / WG_COLS;
+  if (c >= a.C || t >= a.T) return;
+  // Whether every input is a row of this step is known from two entries of row_req (a request's rows are contiguous), and
+  // the TAPS rows before and at t exist whichever request they belong to: all of the thread's loads go out together.
+  const int r = a.row_req[t], r_back = a.row_req[max(t - (TAPS - 1), 0)];
   const bf16_t* x = (const bf16_t*)a.x;
   conv_bf16x8 wv[TAPS], xv[TAPS];       // weights [8 channels][TAPS] as one run; inputs of tap j for the eight channels
 #pragma unroll
   for (int j = 0; j < TAPS; ++j) wv[j] = *(const conv_bf16x8*)((const bf16_t*)a.w + (size_t)c * TAPS + 8 * j);
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) xv[j] = *(const conv_bf16x8*)(x + (size_t)max(t - (TAPS - 1) + j, 0) * a.ld + c);
   float acc[8];
   if (a.b) {
     const conv_bf16x8 b8 = *(const conv_bf16x8*)((const bf16_t*)a.b + c);
@@ -75,14 +84,13 @@ __global__ __launch_bounds__(256) void conv_silu_vec_kernel(ConvArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   }
-  if (i >= TAPS - 1) {       // every input is a row of this step: the usual case
-#pragma unroll
-    for (int j = 0; j < TAPS; ++j) xv[j] = *(const conv_bf16x8*)(x + (size_t)(t - (TAPS - 1) + j) * a.ld + c);
+  if (t >= TAPS - 1 && r_back == r) {       // every input is a row of this step: the usual case
 #pragma unroll
     for (int j = 0; j < TAPS; ++j)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = fmaf((float)wv[(e * TAPS + j) / 8][(e * TAPS + j) % 8], (float)xv[j][e], acc[e]);
   } else {
+    const int t0 = a.q_start[r], i = t - t0;
     const float* st = a.state + (size_t)a.slots[r] * a.state_stride + (size_t)c * (TAPS - 1);
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) {
@@ -140,7 +148,7 @@ extern "C" int ifx_causal_conv(const void* x, int dtype, int ld, const void* w, 
   } else if (dtype == DT_BF16) {
     // (many rows only: a thread of eight channels leaves a step of few rows too few threads to fill the chip)
     const bool vec = C % 8 == 0 && ld % 8 == 0 && w_dtype == DT_BF16 && (long long)T * C >= (1 << 20);
-    const dim3 vgrid((unsigned)((C / 8 + 255) / 256), T);
+    const dim3 vgrid((unsigned)((C / 8 + 256 / CONV_WG_ROWS - 1) / (256 / CONV_WG_ROWS)), (unsigned)((T + CONV_WG_ROWS - 1) / CONV_WG_ROWS));
     if (vec && taps == 4) hipLaunchKernelGGL(conv_silu_vec_kernel<4>, vgrid, dim3(256), 0, s, a);
     else if (vec && taps == 3) hipLaunchKernelGGL(conv_silu_vec_kernel<3>, vgrid, dim3(256), 0, s, a);
     else if (vec && taps == 2) hipLaunchKernelGGL(conv_silu_vec_kernel<2>, vgrid, dim3(256), 0, s, a);
