@@ -94,8 +94,8 @@ class PagedAttention(Mixer):
             out[nm["v_bias"]] = ParamSpec((self.n_kv_heads * dv,), s)
         if self.output_gate:
             out[nm["gate"]] = ParamSpec((self.n_heads, H), s)
-        if self.value_mix is not None:       # (the source layer's tensor is in the file too; nothing reads it)
-            out[nm["mix"]] = ParamSpec((), ("uniform", 0.2, 0.8))
+        if self.value_mix is not None:       # (the source layer's tensor is in the file too, where the file has it; nothing reads it)
+            out[nm["mix"]] = ParamSpec((), ("uniform", 0.2, 0.8), optional=self.value_mix == "source")
         return out
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:

@@ -614,6 +614,30 @@ def test_replay_of_traces_with_pages_and_slots_used_again(name, dtype, folders, 
         assert rel_err(got, want) < TOL[dtype], (step, rows[:3])
 
 
+def test_replay_takes_a_file_with_tensors_nobody_reads(folders, tmp_path):
+    """A model file may hold more than the model reads (a second norm in a layer without feed-forward) and less where a
+    tensor is read by nobody (the first mixing layer's weight): the replay tool lists the former and goes on, unless told to
+    be strict; the logits are the same."""
+    from safetensors.torch import load_file, save_file
+    import shutil
+    src = folders["B", "float32"]
+    folder = str(tmp_path / "m")
+    shutil.copytree(src, folder)
+    t = load_file(os.path.join(folder, "model.safetensors"))
+    t["l2.norm2"] = torch.ones(88, dtype=torch.bfloat16)           # layer 2 has no feed-forward
+    del t["l1.mix.vmix"]                                           # the one mixing layer hands its values on and mixes nothing
+    save_file(t, os.path.join(folder, "model.safetensors"))
+    ids = ids_of(95, 40, 131)
+    step = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": ids, "want": [39]}], "end": ["a"]}) + "\n"
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--max-tokens", "64"]
+    ok = subprocess.run(cmd + ["--out", str(tmp_path / "o1")], input=step, capture_output=True, text=True, timeout=120)
+    assert ok.returncode == 0 and "done 0" in ok.stdout and "l2.norm2" in ok.stderr
+    got = torch.from_numpy(np.fromfile(str(tmp_path / "o1" / "0.f32"), dtype="<f4"))
+    assert rel_err(got[None], plain(src, ids)[39:40]) < TOL["float32"]
+    strict = subprocess.run(cmd + ["--out", str(tmp_path / "o2"), "--strict-weights"], input=step, capture_output=True, text=True, timeout=120)
+    assert strict.returncode != 0 and "l2.norm2" in strict.stderr
+
+
 def _drawn_config(seed):
     """A configuration drawn from sizes of every kind: heads the matrix-core kernels take and heads only the plain kernel
     takes, grouped and ungrouped, values wider and narrower than keys, windows around a page's size with and without
